@@ -341,6 +341,127 @@ class LusolixConfig:
                     raise ConfigError(f"layers[{i}]: {mlp['top']} of {mlp['experts']} experts")
 
 
+@dataclass(frozen=True)
+class GaboraxLayer:
+    """One entry of a Gaborax model's list of layers."""
+    type: str                                  # "attention" | "attention_2"
+    mixer: dict                                # the mixer's sizes and constants, as config.json gives them
+    mlp: dict | None                           # {"ff", "experts", "identity", "top", "shared_ff"} | None
+
+
+@dataclass(frozen=True)
+class GaboraxConfig:
+    """The Gaborax decoder: token embedding; layers whose sublayers read the residual stream itself and whose results pass
+    an RMS norm (weight stored around zero) and a per-channel layer scale on their way into it; softmax attention with q and
+    k normed over the whole projection, in two kinds (``attention``: rotation of half-apart pairs, a gate per head, possibly
+    on another layer's keys and values; ``attention_2``: biases, rotation of neighbouring pairs with scaled frequencies,
+    capped scores); a feed-forward of routed experts (relu squared, experts that stand for the input, a gated shared
+    expert); the output head is the embedding table. Every size and constant that can differ between two models is read
+    from config.json; the model has no position limit of its own (``max_positions`` if the file gives one)."""
+
+    vocab_size: int
+    hidden_size: int
+    norm_eps: float
+    layers: tuple[GaboraxLayer, ...]
+    max_position_embeddings: int | None = None
+    eos_token_ids: tuple[int, ...] = field(default_factory=tuple)
+
+    architecture = "Gaborax"
+    MIXERS = ("attention", "attention_2")
+
+    @property
+    def num_hidden_layers(self) -> int:
+        return len(self.layers)
+
+    @classmethod
+    def from_dict(cls, raw: dict, generation: dict | None = None) -> "GaboraxConfig":
+        norm = _require(raw, "norm")
+        layers = []
+        for i, entry in enumerate(_require(raw, "layers")):
+            kind = entry.get("type")
+            if kind not in cls.MIXERS:
+                raise ConfigError(f"layers[{i}]: type '{kind}' is not one of {list(cls.MIXERS)}")
+            mixer = entry.get("mixer")
+            if not isinstance(mixer, dict):
+                raise ConfigError(f"layers[{i}] has no 'mixer' sizes")
+            for key in ("heads", "dim", "vdim", "scale"):
+                if mixer.get(key) is None:
+                    raise ConfigError(f"layers[{i}]: the {kind} mixer has no '{key}'")
+            mlp = entry.get("mlp")
+            if mlp is not None:
+                how = mlp.get("kind", "moe")
+                if how != "moe":
+                    raise ConfigError(f"layers[{i}]: feed-forward kind '{how}' is not 'moe'")
+                expert, router, shared = mlp.get("expert") or {}, mlp.get("router") or {}, mlp.get("shared")
+                for where, key in ((router, "experts"), (router, "top")):
+                    if where.get(key) is None:
+                        raise ConfigError(f"layers[{i}]: the experts have no '{key}'")
+                if int(router["experts"]) > 0 and expert.get("ff") is None:
+                    raise ConfigError(f"layers[{i}]: the experts have no 'ff' width")
+                mlp = {"ff": int(expert.get("ff") or 0), "experts": int(router["experts"]), "identity": int(router.get("identity") or 0),
+                       "top": int(router["top"]), "shared_ff": int(shared["ff"]) if shared and shared.get("ff") else None}
+            layers.append(GaboraxLayer(kind, dict(mixer), mlp))
+        most = raw.get("max_positions")
+        cfg = cls(vocab_size=int(_require(raw, "vocab")), hidden_size=int(_require(raw, "width")), norm_eps=float(_require(norm, "eps")),
+                  layers=tuple(layers), max_position_embeddings=int(most) if most is not None else None,
+                  eos_token_ids=collect_eos_ids(([generation] if generation else []) + [raw]))
+        cfg.validate()
+        return cfg
+
+    def validate(self) -> None:
+        for name in ("vocab_size", "hidden_size"):
+            if getattr(self, name) <= 0:
+                raise ConfigError(f"{name} must be positive, got {getattr(self, name)}")
+        if self.max_position_embeddings is not None and self.max_position_embeddings <= 0:
+            raise ConfigError("max_positions must be positive")
+        if not self.norm_eps > 0:
+            raise ConfigError("norm.eps must be positive")
+        if not self.layers:
+            raise ConfigError("a model needs at least one layer")
+        for i, layer in enumerate(self.layers):
+            m = layer.mixer
+            for key in ("heads", "dim", "vdim"):
+                if int(m[key]) <= 0:
+                    raise ConfigError(f"layers[{i}]: {key} must be positive")
+            heads, kv = int(m["heads"]), int(m.get("kv_heads") or m["heads"])
+            if kv <= 0 or heads % kv:
+                raise ConfigError(f"layers[{i}]: {heads} heads do not divide into {kv} kv_heads")
+            rot = m.get("rot")
+            if rot:
+                dims = int(rot.get("dims", 0))
+                if dims < 0 or dims % 2 or dims > int(m["dim"]):
+                    raise ConfigError(f"layers[{i}]: rot.dims {dims} must be even and at most dim {m['dim']}")
+                if dims and not float(rot.get("base", 0)) > 0:
+                    raise ConfigError(f"layers[{i}]: rot.base must be positive")
+                sc = rot.get("scaling")
+                if sc:
+                    for key in ("factor", "original", "fast", "slow"):
+                        if sc.get(key) is None or not float(sc[key]) > 0:
+                            raise ConfigError(f"layers[{i}]: rot.scaling.{key} must be positive")
+            if m.get("softcap") is not None and not float(m["softcap"]) > 0:
+                raise ConfigError(f"layers[{i}]: softcap must be positive")
+            src = m.get("kv_from")
+            if src is not None:
+                if layer.type != "attention":
+                    raise ConfigError(f"layers[{i}]: only an 'attention' mixer reads another layer's keys and values")
+                src = int(src)
+                if not 0 <= src < i or self.layers[src].mixer.get("kv_from") is not None:
+                    raise ConfigError(f"layers[{i}]: kv_from must name an earlier layer that has keys and values of its own")
+                other = self.layers[src].mixer
+                same = all(int(other.get(k) or other["heads"]) == int(m.get(k) or m["heads"]) for k in ("kv_heads",)) and \
+                    all(int(other[k]) == int(m[k]) for k in ("heads", "dim", "vdim")) and (other.get("rot") or {}) == (m.get("rot") or {})
+                if not same:
+                    raise ConfigError(f"layers[{i}]: layer {src}'s head counts, sizes and rotation must equal this layer's")
+            mlp = layer.mlp
+            if mlp is not None:
+                if mlp["experts"] < 0 or mlp["identity"] < 0 or not 0 < mlp["top"] <= mlp["experts"] + mlp["identity"]:
+                    raise ConfigError(f"layers[{i}]: {mlp['top']} of {mlp['experts']} + {mlp['identity']} experts")
+                if mlp["experts"] and mlp["ff"] <= 0:
+                    raise ConfigError(f"layers[{i}]: expert.ff must be positive")
+                if mlp["shared_ff"] is not None and mlp["shared_ff"] <= 0:
+                    raise ConfigError(f"layers[{i}]: shared.ff must be positive")
+
+
 def read_json(path: Path) -> dict:
     try:
         return json.loads(path.read_text())

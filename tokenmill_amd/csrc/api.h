@@ -41,6 +41,20 @@ int tm_attn_paged_generic(const void* q, int q_stride, void* out, int out_stride
                           const int* positions, int T, int H, int KVH, int D, int page, float scale, int window,
                           int dtype, hipStream_t stream);
 
+// The same with keys and values of different sizes (D, DV), scores capped smoothly at +-softcap (0: as they are) and a gate
+// per (token, head) (float32, rows ldg apart; null: none) whose sigmoid multiplies the head's result.
+int tm_attn_paged_generic_ext(const void* q, int q_stride, void* out, int out_stride, const void* k_pool, const void* v_pool,
+                              const int* block_tables, int table_width, const int* seq_of_token, const int* positions, int T, int H,
+                              int KVH, int D, int DV, int page, float scale, int window, float softcap, const float* gate, int ldg,
+                              int dtype, hipStream_t stream);
+
+// q and k normed over the whole projection, rotated and stored (attention_prepare.hip): see the head of that file.
+int tm_whole_norm_rope_store(const float* proj, int ld, void* q_out, int dtype, int T, int H, int G, int D, int Dv, int rot,
+                             int interleaved, const float* q_w, const float* k_w, float eps, const float* cos_t, const float* sin_t,
+                             const int* positions, const int* slots, void* k_pool, void* v_pool, int page, int has_kv,
+                             hipStream_t stream);
+int tm_head_gate(void* x, int dtype, const float* gate, int ldg, int T, int H, int Dv, hipStream_t stream);
+
 int tm_gemm_skinny(const void* A, int lda, const void* W, const void* bias, int bias_dtype, void* C, int ldc, int M,
                    int N, int K, int out_dtype, int silu, float* accum, int ldacc, hipStream_t stream);
 
@@ -123,6 +137,7 @@ int tm_embed_gather_pos(const void* table, const void* places, int dtype, const 
                         float* out, int T, int hidden, int vocab, int max_pos, hipStream_t stream);
 
 int tm_gelu_tanh(const void* in, void* out, int dtype, long long n, hipStream_t stream);
+int tm_relu2(const void* in, void* out, int dtype, long long n, hipStream_t stream);
 
 // RMS norm in `groups` equal consecutive parts of a row, around a sublayer (norm_groups.hip):
 // resid[r] += norm(y[r]; post_w) (post_w null: y as it is; y null: nothing), out[r] = norm(resid[r]; pre_w) (out null: none).
@@ -217,6 +232,18 @@ int tm_moe_down(const void* act, const void* W, float* part, const int* tiles, c
                 int dtype, hipStream_t stream);
 int tm_moe_combine(const float* part, const int* pair_slot, void* y, int T, int top, float weight, int N, int dtype,
                    hipStream_t stream);
+
+// Experts chosen by a router, experts without a gate, experts that stand for the input itself, a shared expert (moe.hip).
+int tm_moe_router(const float* z, int ldz, const float* correction, int T, int E, int top, int* chosen, float* weight,
+                  hipStream_t stream);
+int tm_moe_route_chosen(const int* ids, const int* table, int T, int top, int E, int real, int tile_rows, int* slot_pair,
+                        int* pair_slot, int* tiles, int* n_tiles, hipStream_t stream);
+int tm_moe_up_act(const void* x, int ldx, const int* slot_pair, int top, const void* W, void* act, const int* tiles,
+                  const int* n_tiles, int max_tiles, int K, int F, int dtype, hipStream_t stream);
+int tm_moe_combine_weighted(const float* part, const int* pair_slot, const float* weight, const void* x, int ldx, const float* shared,
+                            const float* shared_gate, int ldg, void* y, int T, int top, int N, int dtype, hipStream_t stream);
+int tm_moe_up_act_mfma(const void* x, int ldx, const int* slot_pair, int top, const void* W, void* act, const int* tiles,
+                       const int* n_tiles, int max_tiles, int tile_rows, int K, int F, hipStream_t stream);
 
 // The per-head products and the experts' products on the matrix unit (grouped_mfma.hip), bfloat16; the matrices as
 // [groups, N, K] with k contiguous. The *_takes functions say whether the operands come in whole 16-byte pieces.

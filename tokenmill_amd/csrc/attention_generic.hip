@@ -37,6 +37,9 @@ __device__ __forceinline__ void ag_load4(const bf16_t* p, float (&v)[4]) {
     v[3] = __uint_as_float(t.y & 0xffff0000u);
 }
 
+// scores capped smoothly at +-cap (0: as they are)
+__device__ __forceinline__ float ag_capped(float sc, float cap) { return cap > 0.f ? cap * tanhf(sc / cap) : sc; }
+
 // SPLIT = false: a block is AG_WAVES (token, head) pairs, one per wavefront (steps with many tokens).
 // SPLIT = true : a block is one (token, head) pair; its AG_SPLIT_WAVES wavefronts take the groups of 64
 //                keys in turn (group i goes to wavefront i % AG_SPLIT_WAVES) and their partial results
@@ -52,7 +55,7 @@ __global__ __launch_bounds__((SPLIT ? AG_SPLIT_WAVES : AG_WAVES) * TM_WAVE) void
     const T* __restrict__ q, int q_stride, T* __restrict__ out, int out_stride,
     const T* __restrict__ k_pool, const T* __restrict__ v_pool, const int* __restrict__ block_tables,
     int table_width, const int* __restrict__ seq_of_token, const int* __restrict__ positions, int T_tokens,
-    int H, int KVH, int D, int page, float scale, int window) {
+    int H, int KVH, int D, int DV, int page, float scale, int window, float softcap, const float* __restrict__ gate, int ldg) {
     constexpr int WAVES = SPLIT ? AG_SPLIT_WAVES : AG_WAVES;
     constexpr bool STAGED = DMAX > 0 && sizeof(T) == 4;         // 32-bit keys through LDS (see the key loop)
     __shared__ __align__(16) float k_tile[STAGED ? WAVES : 1][STAGED ? TM_WAVE * AG_KSTRIDE : 4];
@@ -129,7 +132,7 @@ __global__ __launch_bounds__((SPLIT ? AG_SPLIT_WAVES : AG_WAVES) * TM_WAVE) void
                     }
                 }
             }
-            if (valid) sc = dot * scale;
+            if (valid) sc = ag_capped(dot * scale, softcap);
         } else if (valid) {
             row = (long long)table[j / page] * page + (j % page);
             const T* kr = k_pool + ((size_t)row * KVH + kvh) * D;
@@ -142,7 +145,7 @@ __global__ __launch_bounds__((SPLIT ? AG_SPLIT_WAVES : AG_WAVES) * TM_WAVE) void
                 dot = fmaf(qs[d + 2], kv[2], dot);
                 dot = fmaf(qs[d + 3], kv[3], dot);
             }
-            sc = dot * scale;
+            sc = ag_capped(dot * scale, softcap);
         }
         const float m_new = fmaxf(m, wave_max(sc));     // finite: lane 0 of every group is valid
         const float corr = expf(m - m_new);             // exp(-inf) = 0 on the first group
@@ -153,14 +156,14 @@ __global__ __launch_bounds__((SPLIT ? AG_SPLIT_WAVES : AG_WAVES) * TM_WAVE) void
         if constexpr (DMAX > 0) {
             // a lane beyond the newest key reads the newest key's values (finite) with weight 0
             const long long rv = (valid || STAGED) ? row : (long long)table[p / page] * page + (p % page);
-            const T* vr = v_pool + ((size_t)(rv / page) * KVH + kvh) * D * page + (rv % page);
+            const T* vr = v_pool + ((size_t)(rv / page) * KVH + kvh) * DV * page + (rv % page);
             // every load without a test, all of a group in flight at once: beyond D a lane reads d = 0
             // again and the sum it feeds is never looked at
 #pragma unroll
             for (int d0 = 0; d0 < DMAX; d0 += 64) {     // 64 loads in flight at a time
                 float vals[64];
 #pragma unroll
-                for (int d = 0; d < 64; ++d) vals[d] = Elem<T>::load(vr + (size_t)(d0 + d < D ? d0 + d : 0) * page);
+                for (int d = 0; d < 64; ++d) vals[d] = Elem<T>::load(vr + (size_t)(d0 + d < DV ? d0 + d : 0) * page);
                 __builtin_amdgcn_sched_barrier(0);      // (else the compiler asks for them one by one, to save registers)
 #pragma unroll
                 for (int d = 0; d < 64; ++d) part[d0 + d] = fmaf(pr_v, vals[d], part[d0 + d] * corr);
@@ -174,30 +177,32 @@ __global__ __launch_bounds__((SPLIT ? AG_SPLIT_WAVES : AG_WAVES) * TM_WAVE) void
         for (int jj = 0; jj < n; ++jj) {
             const float pj = __shfl(pr_v, jj, TM_WAVE);
             const long long rj = __shfl(row, jj, TM_WAVE);
-            const T* vr = v_pool + ((size_t)(rj / page) * KVH + kvh) * D * page + (rj % page);
+            const T* vr = v_pool + ((size_t)(rj / page) * KVH + kvh) * DV * page + (rj % page);
 #pragma unroll
             for (int i = 0; i < AG_MAXD / TM_WAVE; ++i) {
                 const int d = lane + i * TM_WAVE;
-                if (d < D) acc[i] = fmaf(pj, Elem<T>::load(vr + (size_t)d * page), acc[i]);
+                if (d < DV) acc[i] = fmaf(pj, Elem<T>::load(vr + (size_t)d * page), acc[i]);
             }
         }
     }
     if constexpr (DMAX > 0) {                   // the lanes' sums added, lane d % 64 keeps d
 #pragma unroll
         for (int d = 0; d < DMAX; ++d) {
-            if (d < D) {
+            if (d < DV) {
                 const float total = wave_sum(part[d]);
                 if (lane == d % TM_WAVE) acc[d / TM_WAVE] = total;
             }
         }
     }
-    T* orow = out + (size_t)t * out_stride + (size_t)h * D;
+    T* orow = out + (size_t)t * out_stride + (size_t)h * DV;
+    // a gate per (token, head): the result times the sigmoid of the gate's 32-bit value, before its one rounding
+    const float gated = gate ? 1.f / (1.f + expf(-gate[(size_t)t * ldg + h])) : 1.f;
     if (!SPLIT) {
-        const float inv = 1.f / l;
+        const float inv = gated / l;
 #pragma unroll
         for (int i = 0; i < AG_MAXD / TM_WAVE; ++i) {
             const int d = lane + i * TM_WAVE;
-            if (d < D) Elem<T>::store(orow + d, acc[i] * inv);
+            if (d < DV) Elem<T>::store(orow + d, acc[i] * inv);
         }
         return;
     }
@@ -209,7 +214,7 @@ __global__ __launch_bounds__((SPLIT ? AG_SPLIT_WAVES : AG_WAVES) * TM_WAVE) void
 #pragma unroll
     for (int i = 0; i < AG_MAXD / TM_WAVE; ++i) {
         const int d = lane + i * TM_WAVE;
-        if (d < D) s_acc[wave][d] = acc[i];
+        if (d < DV) s_acc[wave][d] = acc[i];
     }
     __syncthreads();
     float mm = s_m[0];
@@ -218,65 +223,78 @@ __global__ __launch_bounds__((SPLIT ? AG_SPLIT_WAVES : AG_WAVES) * TM_WAVE) void
     float ll = 0.f;
 #pragma unroll
     for (int ww = 0; ww < WAVES; ++ww) ll += (s_m[ww] == -INFINITY) ? 0.f : s_l[ww] * expf(s_m[ww] - mm);
-    for (int d = threadIdx.x; d < D; d += WAVES * TM_WAVE) {
+    for (int d = threadIdx.x; d < DV; d += WAVES * TM_WAVE) {
         float oo = 0.f;
 #pragma unroll
         for (int ww = 0; ww < WAVES; ++ww) oo += (s_m[ww] == -INFINITY) ? 0.f : s_acc[ww][d] * expf(s_m[ww] - mm);
-        Elem<T>::store(orow + d, oo / ll);
+        Elem<T>::store(orow + d, oo / ll * gated);
     }
 }
 
 template <typename T, int DMAX>
 static void launch_generic_d(const void* q, int q_stride, void* out, int out_stride, const void* k_pool,
                              const void* v_pool, const int* block_tables, int table_width, const int* seq_of_token,
-                             const int* positions, int T_tokens, int H, int KVH, int D, int page, float scale,
-                             int window, hipStream_t stream) {
+                             const int* positions, int T_tokens, int H, int KVH, int D, int DV, int page, float scale,
+                             int window, float softcap, const float* gate, int ldg, hipStream_t stream) {
     const long long pairs = (long long)T_tokens * H;
     if (pairs < 1024)           // too few (token, head) pairs to fill the chip: the wavefronts of a block split the keys
         attn_paged_generic_kernel<T, true, DMAX><<<(unsigned)pairs, AG_SPLIT_WAVES * TM_WAVE, 0, stream>>>(
             (const T*)q, q_stride, (T*)out, out_stride, (const T*)k_pool, (const T*)v_pool, block_tables,
-            table_width, seq_of_token, positions, T_tokens, H, KVH, D, page, scale, window);
+            table_width, seq_of_token, positions, T_tokens, H, KVH, D, DV, page, scale, window, softcap, gate, ldg);
     else
         attn_paged_generic_kernel<T, false, DMAX><<<(unsigned)((pairs + AG_WAVES - 1) / AG_WAVES),
                                                     AG_WAVES * TM_WAVE, 0, stream>>>(
             (const T*)q, q_stride, (T*)out, out_stride, (const T*)k_pool, (const T*)v_pool, block_tables,
-            table_width, seq_of_token, positions, T_tokens, H, KVH, D, page, scale, window);
+            table_width, seq_of_token, positions, T_tokens, H, KVH, D, DV, page, scale, window, softcap, gate, ldg);
 }
 
 template <typename T>
 static void launch_generic(const void* q, int q_stride, void* out, int out_stride, const void* k_pool,
                            const void* v_pool, const int* block_tables, int table_width, const int* seq_of_token,
-                           const int* positions, int T_tokens, int H, int KVH, int D, int page, float scale,
-                           int window, hipStream_t stream) {
+                           const int* positions, int T_tokens, int H, int KVH, int D, int DV, int page, float scale,
+                           int window, float softcap, const float* gate, int ldg, hipStream_t stream) {
 #define TM_GENERIC(DMAX)                                                                                       \
     launch_generic_d<T, DMAX>(q, q_stride, out, out_stride, k_pool, v_pool, block_tables, table_width,         \
-                              seq_of_token, positions, T_tokens, H, KVH, D, page, scale, window, stream)
-    if (D <= 64) TM_GENERIC(64);
-    else if (D <= 128) TM_GENERIC(128);
+                              seq_of_token, positions, T_tokens, H, KVH, D, DV, page, scale, window, softcap, gate, ldg, stream)
+    const int widest = D > DV ? D : DV;
+    if (widest <= 64) TM_GENERIC(64);
+    else if (widest <= 128) TM_GENERIC(128);
     else TM_GENERIC(0);
 #undef TM_GENERIC
+}
+
+// D: size of a key, DV: of a value (the V pool is [pages, KVH, DV, page], out rows H * DV); softcap > 0: a score s becomes
+// softcap * tanh(s / softcap); gate (float32 [T, >= H], rows ldg apart) or null: head h of token t is multiplied by
+// sigmoid(gate[t][h]).
+extern "C" int tm_attn_paged_generic_ext(const void* q, int q_stride, void* out, int out_stride, const void* k_pool,
+                                         const void* v_pool, const int* block_tables, int table_width,
+                                         const int* seq_of_token, const int* positions, int T, int H, int KVH, int D, int DV,
+                                         int page, float scale, int window, float softcap, const float* gate, int ldg,
+                                         int dtype, hipStream_t stream) {
+    if (T <= 0) return TM_OK;
+    if (H <= 0 || KVH <= 0 || H % KVH || D <= 0 || D > AG_MAXD || D % 4 || DV <= 0 || DV > AG_MAXD || page <= 0 ||
+        table_width <= 0 || window < 0 || q_stride < H * D || out_stride < H * DV || !(softcap >= 0.f) || (gate && ldg < H))
+        return TM_ERR_ARG;
+    if (((long long)T * H + AG_WAVES - 1) / AG_WAVES > 0x7fffffffLL) return TM_ERR_ARG;
+    if (dtype == TM_F32) {
+        if (((uintptr_t)k_pool % 16)) return TM_ERR_ARG;
+        launch_generic<float>(q, q_stride, out, out_stride, k_pool, v_pool, block_tables, table_width, seq_of_token,
+                              positions, T, H, KVH, D, DV, page, scale, window, softcap, gate, ldg, stream);
+    } else if (dtype == TM_BF16) {
+        if (((uintptr_t)k_pool % 8)) return TM_ERR_ARG;
+        launch_generic<bf16_t>(q, q_stride, out, out_stride, k_pool, v_pool, block_tables, table_width, seq_of_token,
+                               positions, T, H, KVH, D, DV, page, scale, window, softcap, gate, ldg, stream);
+    } else {
+        return TM_ERR_ARG;
+    }
+    TM_CHECK_LAUNCH();
+    return TM_OK;
 }
 
 extern "C" int tm_attn_paged_generic(const void* q, int q_stride, void* out, int out_stride, const void* k_pool,
                                      const void* v_pool, const int* block_tables, int table_width,
                                      const int* seq_of_token, const int* positions, int T, int H, int KVH, int D,
                                      int page, float scale, int window, int dtype, hipStream_t stream) {
-    if (T <= 0) return TM_OK;
-    if (H <= 0 || KVH <= 0 || H % KVH || D <= 0 || D > AG_MAXD || D % 4 || page <= 0 || table_width <= 0 ||
-        window < 0 || q_stride < H * D || out_stride < H * D)
-        return TM_ERR_ARG;
-    if (((long long)T * H + AG_WAVES - 1) / AG_WAVES > 0x7fffffffLL) return TM_ERR_ARG;
-    if (dtype == TM_F32) {
-        if (((uintptr_t)k_pool % 16)) return TM_ERR_ARG;
-        launch_generic<float>(q, q_stride, out, out_stride, k_pool, v_pool, block_tables, table_width, seq_of_token,
-                              positions, T, H, KVH, D, page, scale, window, stream);
-    } else if (dtype == TM_BF16) {
-        if (((uintptr_t)k_pool % 8)) return TM_ERR_ARG;
-        launch_generic<bf16_t>(q, q_stride, out, out_stride, k_pool, v_pool, block_tables, table_width, seq_of_token,
-                               positions, T, H, KVH, D, page, scale, window, stream);
-    } else {
-        return TM_ERR_ARG;
-    }
-    TM_CHECK_LAUNCH();
-    return TM_OK;
+    return tm_attn_paged_generic_ext(q, q_stride, out, out_stride, k_pool, v_pool, block_tables, table_width, seq_of_token,
+                                     positions, T, H, KVH, D, D, page, scale, window, 0.f, nullptr, 0, dtype, stream);
 }

@@ -425,46 +425,68 @@ __device__ __forceinline__ float gelu_tanh_f32(float z) {
     return 0.5f * z * (1.f + tanhf(u));
 }
 
-template <typename T>
-__global__ void gelu_tanh_kernel(const T* __restrict__ in, T* __restrict__ out, size_t n) {
+// the square of relu, also in 32-bit
+__device__ __forceinline__ float relu2_f32(float z) {
+    const float r = fmaxf(z, 0.f);
+    return r * r;
+}
+
+enum { ACT_GELU_TANH = 0, ACT_RELU2 = 1 };
+
+template <int ACT>
+__device__ __forceinline__ float act_f32(float z) { return ACT == ACT_RELU2 ? relu2_f32(z) : gelu_tanh_f32(z); }
+
+template <typename T, int ACT>
+__global__ void activation_kernel(const T* __restrict__ in, T* __restrict__ out, size_t n) {
     for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x)
-        Elem<T>::store(out + i, gelu_tanh_f32(Elem<T>::load(in + i)));
+        Elem<T>::store(out + i, act_f32<ACT>(Elem<T>::load(in + i)));
 }
 
 // bfloat16, eight elements (16 bytes) per thread and step
-__global__ void gelu_tanh_bf16x8_kernel(const bf16_t* __restrict__ in, bf16_t* __restrict__ out, size_t groups) {
+template <int ACT>
+__global__ void activation_bf16x8_kernel(const bf16_t* __restrict__ in, bf16_t* __restrict__ out, size_t groups) {
     for (size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x; idx < groups; idx += (size_t)gridDim.x * blockDim.x) {
         const uint4 v = *(const uint4*)(in + 8 * idx);
         const uint32_t w[4] = {v.x, v.y, v.z, v.w};
         uint32_t o[4];
 #pragma unroll
         for (int k = 0; k < 4; ++k) {
-            const float a = gelu_tanh_f32(__uint_as_float(w[k] << 16)), b = gelu_tanh_f32(__uint_as_float(w[k] & 0xffff0000u));
+            const float a = act_f32<ACT>(__uint_as_float(w[k] << 16)), b = act_f32<ACT>(__uint_as_float(w[k] & 0xffff0000u));
             o[k] = (uint32_t)f32_to_bf16(a) | ((uint32_t)f32_to_bf16(b) << 16);
         }
         *(uint4*)(out + 8 * idx) = uint4{o[0], o[1], o[2], o[3]};
     }
 }
 
-extern "C" int tm_gelu_tanh(const void* in, void* out, int dtype, long long n, hipStream_t stream) {
+template <int ACT>
+static int launch_activation(const void* in, void* out, int dtype, long long n, hipStream_t stream) {
     if (n <= 0) return TM_OK;
     if (!in || !out) return TM_ERR_ARG;
     if (dtype == TM_BF16 && n % 8 == 0 && ((uintptr_t)in % 16) == 0 && ((uintptr_t)out % 16) == 0) {
         const size_t groups = (size_t)n / 8, want = (groups + 255) / 256;
-        gelu_tanh_bf16x8_kernel<<<(int)(want < 65536 ? want : 65536), 256, 0, stream>>>((const bf16_t*)in, (bf16_t*)out, groups);
+        activation_bf16x8_kernel<ACT><<<(int)(want < 65536 ? want : 65536), 256, 0, stream>>>((const bf16_t*)in, (bf16_t*)out, groups);
         TM_CHECK_LAUNCH();
         return TM_OK;
     }
     const size_t want = ((size_t)n + 255) / 256;
     const int blocks = (int)(want < 16384 ? want : 16384);
     if (dtype == TM_F32)
-        gelu_tanh_kernel<float><<<blocks, 256, 0, stream>>>((const float*)in, (float*)out, (size_t)n);
+        activation_kernel<float, ACT><<<blocks, 256, 0, stream>>>((const float*)in, (float*)out, (size_t)n);
     else if (dtype == TM_BF16)
-        gelu_tanh_kernel<bf16_t><<<blocks, 256, 0, stream>>>((const bf16_t*)in, (bf16_t*)out, (size_t)n);
+        activation_kernel<bf16_t, ACT><<<blocks, 256, 0, stream>>>((const bf16_t*)in, (bf16_t*)out, (size_t)n);
     else
         return TM_ERR_ARG;
     TM_CHECK_LAUNCH();
     return TM_OK;
+}
+
+extern "C" int tm_gelu_tanh(const void* in, void* out, int dtype, long long n, hipStream_t stream) {
+    return launch_activation<ACT_GELU_TANH>(in, out, dtype, n, stream);
+}
+
+// out[i] = relu(in[i])^2 (in place allowed)
+extern "C" int tm_relu2(const void* in, void* out, int dtype, long long n, hipStream_t stream) {
+    return launch_activation<ACT_RELU2>(in, out, dtype, n, stream);
 }
 
 // ------------------------------------------------------------------------------------------

@@ -5,7 +5,7 @@
 //   experts : tiles (group, first slot, rows <= 32) from tm_moe_route; a tile's rows are slots first .. first + rows - 1, and
 //             slot i reads row row_src[i] / src_div of A (row_src null: row i).
 // Epilogues: a plain store in bfloat16 or in 32-bit, or, with a matrix of 2 N rows (gate rows, then up rows),
-// silu(gate product) * up product. A block is RT tiles of 16 rows by 64 columns; its four wavefronts take 16 columns each;
+// silu(gate product) * up product, or the square of relu(product) in bfloat16. A block is RT tiles of 16 rows by 64 columns; its four wavefronts take 16 columns each;
 // k ascends in steps of 32 through LDS, so an element's sum has one order wherever its row stands.
 #include "common.h"
 #include "api.h"
@@ -15,7 +15,7 @@
 #define GM_BK 32
 #define GM_LD (GM_BK + 8)
 
-enum { GM_STORE = 0, GM_STORE_F32 = 1, GM_SILU_MUL = 2 };
+enum { GM_STORE = 0, GM_STORE_F32 = 1, GM_SILU_MUL = 2, GM_RELU2 = 3 };
 
 template <int RT, int MODE>
 __global__ __launch_bounds__(256) void grouped_mfma_kernel(const bf16_t* __restrict__ A, int lda, int a_off,
@@ -127,6 +127,9 @@ __global__ __launch_bounds__(256) void grouped_mfma_kernel(const bf16_t* __restr
             if (MODE == GM_SILU_MUL) {
                 const float u = acu[t][i];
                 ((bf16_t*)Cv)[at] = f32_to_bf16(v / (1.0f + __expf(-v)) * u);
+            } else if (MODE == GM_RELU2) {
+                v = fmaxf(v, 0.f);
+                ((bf16_t*)Cv)[at] = f32_to_bf16(v * v);
             } else if (MODE == GM_STORE_F32) {
                 ((float*)Cv)[at] = v;
             } else {
@@ -180,6 +183,25 @@ extern "C" int tm_moe_gate_up_mfma(const void* x, int ldx, const int* slot_pair,
 #define GM_GO(RT_)                                                                                                             \
     grouped_mfma_kernel<RT_, GM_SILU_MUL><<<grid, 256, 0, stream>>>((const bf16_t*)x, ldx, 0, slot_pair, top, (const bf16_t*)W, act, F, \
                                                                     0, nullptr, 0, tiles, n_tiles, 0, K, F, 0, 0, nullptr, nullptr, nullptr)
+    if (tile_rows == 32) GM_GO(2); else if (tile_rows == 64) GM_GO(4); else GM_GO(8);
+#undef GM_GO
+    TM_CHECK_LAUNCH();
+    return TM_OK;
+}
+
+// Experts without a gate: act[slot] = relu(x[t] . W[e]^T)^2, W [E, F, K].
+extern "C" int tm_moe_up_act_mfma(const void* x, int ldx, const int* slot_pair, int top, const void* W, void* act, const int* tiles,
+                                  const int* n_tiles, int max_tiles, int tile_rows, int K, int F, hipStream_t stream) {
+    if (tile_rows != 32 && tile_rows != 64 && tile_rows != 128) return TM_ERR_ARG;
+    if (!x || !slot_pair || !W || !act || !tiles || !n_tiles || top <= 0 || K <= 0 || F <= 0 || ldx < K || max_tiles < 0 || K % 8 ||
+        ldx % 8 || !gm_aligned(x) || !gm_aligned(W))
+        return TM_ERR_ARG;
+    if (max_tiles == 0) return TM_OK;
+    dim3 grid(max_tiles, (F + GM_BN - 1) / GM_BN);
+    if (grid.y > 65535) return TM_ERR_ARG;
+#define GM_GO(RT_)                                                                                                             \
+    grouped_mfma_kernel<RT_, GM_RELU2><<<grid, 256, 0, stream>>>((const bf16_t*)x, ldx, 0, slot_pair, top, (const bf16_t*)W, act, F, \
+                                                                 0, nullptr, 0, tiles, n_tiles, 0, K, F, 0, 0, nullptr, nullptr, nullptr)
     if (tile_rows == 32) GM_GO(2); else if (tile_rows == 64) GM_GO(4); else GM_GO(8);
 #undef GM_GO
     TM_CHECK_LAUNCH();

@@ -4,7 +4,8 @@
 //   norm_g(v)[c] = w[c] * v[c] / sqrt(mean(v[group of c]^2) + eps)     the row cut into `groups` equal consecutive parts
 //
 //   resid[r] += norm_g(y[r]; post_w)     (post_w == nullptr: y is added as it is; y == nullptr: nothing is added)
-//   out[r]    = norm_g(resid[r]; pre_w)  (out == nullptr: no second norm)
+//   out[r]    = norm_g(resid[r]; pre_w)  (out == nullptr: no second norm; pre_w == nullptr: out[r] = resid[r], rounded,
+//                                         for a sublayer that reads the residual stream as it is)
 //
 // rows == nullptr: every row, the residual updated in place. rows != nullptr: row rows[r] is read, nothing is written
 // back, out row r (the rows whose logits are wanted).
@@ -98,6 +99,11 @@ __global__ __launch_bounds__(GN_THREADS) void group_norm_kernel(float* __restric
         }
     }
     if (!out) return;
+    if (!pre_w) {                               // the sum itself in the result's type (a thread reads what it wrote)
+        T* o = out + (size_t)r * hidden;
+        for (int c = threadIdx.x; c < hidden; c += GN_THREADS) Elem<T>::store(o + c, xs[c]);
+        return;
+    }
     __syncthreads();
     unit_sums([&](int c) { return xs[c]; }, part, glen, split, units);
     __syncthreads();
@@ -214,6 +220,13 @@ __global__ __launch_bounds__(GN_THREADS) void group_norm_reg_kernel(float* __res
         }
     }
     if (!out) return;
+    if (!pre_w) {
+        T* o = out + (size_t)r * hidden;
+#pragma unroll
+        for (int i = 0; i < GN_PIECES; ++i)
+            if (grp[i] >= 0) GnVec<T>::store(o + 4 * (threadIdx.x + i * GN_THREADS), xv[i]);
+        return;
+    }
 #pragma unroll
     for (int i = 0; i < GN_PIECES; ++i)
         sums[i] = xv[i][0] * xv[i][0] + xv[i][1] * xv[i][1] + xv[i][2] * xv[i][2] + xv[i][3] * xv[i][3];
@@ -263,7 +276,7 @@ extern "C" int tm_group_norm(float* resid, const void* y, const void* post_w, co
                              hipStream_t stream) {
     if (R <= 0) return TM_OK;
     if (hidden <= 0 || groups <= 0 || hidden % groups || !(eps > 0.f) || !resid) return TM_ERR_ARG;
-    if ((out == nullptr) != (pre_w == nullptr)) return TM_ERR_ARG;
+    if (pre_w && !out) return TM_ERR_ARG;
     if (!y && post_w) return TM_ERR_ARG;
     const int split = groups >= GN_WAVES ? 1 : GN_WAVES / groups;
     const size_t lds = ((size_t)hidden + (size_t)groups * split + groups) * sizeof(float);

@@ -1010,6 +1010,15 @@ def gelu_tanh(x: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
     return out
 
 
+def relu2(x: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    """out = relu(x)^2, computed in 32-bit; ``out`` may be ``x``."""
+    _gpu(x, out)
+    _need(x.is_contiguous() and out.is_contiguous() and x.shape == out.shape and x.dtype == out.dtype,
+          "relu2: x and out must be contiguous, of one shape and type")
+    _check(library().tm_relu2(_p(x), _p(out), code(x.dtype), c_longlong(x.numel()), _stream()), "relu2")
+    return out
+
+
 # -------------------------------------------------------------------------------------------- norm in groups
 
 GROUP_NORM_MAX_FLOATS = 16384 - 64        # what a row and its group sums may take of a block's 64 KiB of LDS
@@ -1019,7 +1028,7 @@ def group_norm(resid: torch.Tensor, y: torch.Tensor | None, post_w: torch.Tensor
                out: torch.Tensor | None, groups: int, eps: float, rows: torch.Tensor | None = None) -> torch.Tensor | None:
     """RMS norm in ``groups`` equal consecutive parts of a row, around a sublayer:
     resid += norm(y; post_w) (``post_w`` None: y as it is; ``y`` None: nothing is added), then
-    out = norm(resid; pre_w) (``out`` None: no second norm). With ``rows``: only those rows, out row r from resid row
+    out = norm(resid; pre_w) (``out`` None: no second norm; ``pre_w`` None with an ``out``: out = resid, rounded). With ``rows``: only those rows, out row r from resid row
     rows[r], and resid is not written. resid float32 [T, hidden]; y, out of the model's type; weights [hidden]."""
     _gpu(resid, y, post_w, pre_w, out, rows)
     T, hidden = resid.shape
@@ -1027,7 +1036,7 @@ def group_norm(resid: torch.Tensor, y: torch.Tensor | None, post_w: torch.Tensor
     _need(resid.dtype == torch.float32 and resid.is_contiguous(), "group_norm: the residual stream is contiguous float32")
     _need(groups >= 1 and hidden % groups == 0, f"group_norm: {groups} groups do not divide the width {hidden}")
     _need(hidden + 5 * groups <= GROUP_NORM_MAX_FLOATS, f"group_norm: a row of {hidden} does not fit the kernel's LDS")
-    _need((out is None) == (pre_w is None), "group_norm: out and its norm's weight come together")
+    _need(pre_w is None or out is not None, "group_norm: a second norm needs somewhere to put its result")
     _need(post_w is None or y is not None, "group_norm: a norm of y needs y")
     dtype = out.dtype if out is not None else y.dtype if y is not None else None
     _need(dtype is not None, "group_norm: nothing to do")
@@ -1649,4 +1658,161 @@ def moe_experts(x: torch.Tensor, routed, w_gate_up: torch.Tensor, w_down: torch.
            "moe_down")
     _check(lib.tm_moe_combine(_p(part), _p(pair_slot), _p(out), c_int(T), c_int(top), c_float(weight), c_int(N), dt, _stream()),
            "moe_combine")
+    return out
+
+
+# -------------------------------------------------------------------------------------------- softmax attention with extras
+
+def whole_norm_rope_store(proj: torch.Tensor, q_out: torch.Tensor, H: int, G: int, D: int, Dv: int, q_w: torch.Tensor | None,
+                          k_w: torch.Tensor | None, eps: float, cos: torch.Tensor | None, sin: torch.Tensor | None, interleaved: bool,
+                          positions: torch.Tensor | None, slots: torch.Tensor | None, k_pool: torch.Tensor | None,
+                          v_pool: torch.Tensor | None, has_kv: bool = True) -> torch.Tensor:
+    """proj float32 [T, >= H*D (+ G*D + G*Dv)]: q (and k) are divided by the root mean square of the whole projection (all
+    heads of a token at once) and multiplied by q_w [H*D] / k_w [G*D] (float32; None: no norm), the first 2 * cos.shape[1]
+    channels of every head rotated by the token's position (pairs (j, j + rot/2), or (2j, 2j + 1) if ``interleaved``); q goes
+    to q_out [T, H*D], k and v to the tokens' cache slots. ``has_kv`` False: the row holds no k and v (a layer that reads
+    another layer's cache)."""
+    _gpu(proj, q_out, q_w, k_w, cos, sin, positions, slots, k_pool, v_pool)
+    T = proj.shape[0]
+    width = H * D + (G * (D + Dv) if has_kv else 0)
+    _need(proj.dtype == torch.float32 and proj.dim() == 2 and proj.stride(1) == 1 and proj.shape[1] >= width,
+          f"whole_norm_rope_store: proj is float32 [T, >= {width}]")
+    _need(tuple(q_out.shape) == (T, H * D) and q_out.is_contiguous(), f"whole_norm_rope_store: q_out is contiguous [T, {H * D}]")
+    for w, n in ((q_w, H * D), (k_w, G * D)):
+        if w is not None:
+            _need(w.dtype == torch.float32 and tuple(w.shape) == (n,) and w.is_contiguous(), f"whole_norm_rope_store: a norm weight is float32 [{n}]")
+    _need(not has_kv or (q_w is None) == (k_w is None), "whole_norm_rope_store: q and k are normed together or not at all")
+    rot = 0
+    if cos is not None:
+        rot = 2 * cos.shape[1]
+        _need(sin is not None and cos.dtype == torch.float32 and sin.dtype == torch.float32 and cos.shape == sin.shape
+              and cos.is_contiguous() and sin.is_contiguous() and rot <= D, "whole_norm_rope_store: cos/sin float32 [max_pos, rot/2], rot <= D")
+        _ints(positions, T, "positions")
+    write = has_kv and k_pool is not None
+    page = 0
+    if write:
+        page = _check_pools_kv(k_pool, v_pool, G, D, Dv, q_out.dtype, "whole_norm_rope_store")
+        _ints(slots, T, "slots")
+    ld = proj.stride(0) if T > 1 else max(width, proj.stride(0))
+    _check(library().tm_whole_norm_rope_store(_p(proj), c_int(ld), _p(q_out), c_int(code(q_out.dtype)), c_int(T), c_int(H), c_int(G),
+                                              c_int(D), c_int(Dv), c_int(rot), c_int(1 if interleaved else 0), _p(q_w), _p(k_w),
+                                              c_float(eps), _p(cos), _p(sin), _p(positions), _p(slots if write else None),
+                                              _p(k_pool if write else None), _p(v_pool if write else None), c_int(page),
+                                              c_int(1 if has_kv else 0), _stream()), "whole_norm_rope_store")
+    return q_out
+
+
+def attn_paged_softmax(q: torch.Tensor, out: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor, block_tables: torch.Tensor,
+                       seq_of_token: torch.Tensor, positions: torch.Tensor, H: int, G: int, D: int, Dv: int, scale: float,
+                       window: int = 0, softcap: float = 0.0, gate: torch.Tensor | None = None) -> torch.Tensor:
+    """Softmax attention of every token of the step over its request's cached keys (its own included), a token and a head a
+    wavefront: keys of D channels, values of Dv; a score s becomes softcap * tanh(s / softcap) if ``softcap`` > 0; head h of
+    token t is multiplied by sigmoid(gate[t, h]) (gate: a float32 view [T, >= H] with unit inner stride; None: no gate).
+    q [T, >= H*D] with unit inner stride, out [T, H*Dv]."""
+    _gpu(q, out, k_pool, v_pool, block_tables, seq_of_token, positions, gate)
+    T = q.shape[0]
+    _need(q.stride(1) == 1 and q.shape[1] >= H * D and out.is_contiguous() and tuple(out.shape) == (T, H * Dv),
+          f"attention: q [T, >={H * D}] unit inner stride, out contiguous [T, {H * Dv}]")
+    _need(q.dtype == out.dtype, "attention: q and out share one type")
+    _need(H % G == 0 and D % 4 == 0 and 0 < D <= 256 and 0 < Dv <= 256, "attention(generic): key size a multiple of 4, sizes up to 256")
+    page = _check_pools_kv(k_pool, v_pool, G, D, Dv, q.dtype, "attention")
+    _need(block_tables.dtype == torch.int32 and block_tables.dim() == 2 and block_tables.is_contiguous(),
+          "attention: block_tables must be contiguous int32 [S, W]")
+    _ints(seq_of_token, T, "seq_of_token")
+    _ints(positions, T, "positions")
+    _need(window >= 0 and softcap >= 0, "attention: window and softcap must be >= 0 (0 = none)")
+    ldg = 0
+    if gate is not None:
+        _need(gate.dtype == torch.float32 and gate.dim() == 2 and gate.shape[0] == T and gate.shape[1] >= H and gate.stride(1) == 1,
+              f"attention: gate is float32 [T, >= {H}]")
+        ldg = gate.stride(0) if T > 1 else max(gate.stride(0), H)
+    q_stride = q.stride(0) if T > 1 else max(q.stride(0), H * D)
+    _check(library().tm_attn_paged_generic_ext(_p(q), c_int(q_stride), _p(out), c_int(H * Dv), _p(k_pool), _p(v_pool), _p(block_tables),
+                                               c_int(block_tables.shape[1]), _p(seq_of_token), _p(positions), c_int(T), c_int(H),
+                                               c_int(G), c_int(D), c_int(Dv), c_int(page), c_float(scale), c_int(window),
+                                               c_float(softcap), _p(gate), c_int(ldg), code(q.dtype), _stream()), "attn_paged_generic_ext")
+    return out
+
+
+# -------------------------------------------------------------------------------------------- experts by router
+
+def moe_router(z: torch.Tensor, experts: int, top: int, correction: torch.Tensor | None = None):
+    """z: float32 view [T, >= experts] (the router's outputs). s = softmax over the first ``experts`` columns; the ``top``
+    largest of s + correction are chosen (descending; of equals the lower index). Returns (chosen int32 [T, top], weight
+    float32 [T, top] = the chosen experts' s divided by their sum + 1e-20)."""
+    _gpu(z, correction)
+    T = z.shape[0]
+    _need(z.dtype == torch.float32 and z.dim() == 2 and z.stride(1) == 1 and z.shape[1] >= experts, f"moe_router: z is float32 [T, >= {experts}]")
+    _need(0 < top <= experts <= MOE_MAX_EXPERTS, f"moe_router: {top} of {experts} experts (up to {MOE_MAX_EXPERTS})")
+    if correction is not None:
+        _need(correction.dtype == torch.float32 and tuple(correction.shape) == (experts,) and correction.is_contiguous(),
+              f"moe_router: correction is float32 [{experts}]")
+    chosen = torch.empty((T, top), dtype=torch.int32, device=z.device)
+    weight = torch.empty((T, top), dtype=torch.float32, device=z.device)
+    ldz = z.stride(0) if T > 1 else max(z.stride(0), experts)
+    _check(library().tm_moe_router(_p(z), c_int(ldz), _p(correction), c_int(T), c_int(experts), c_int(top), _p(chosen), _p(weight),
+                                   _stream()), "moe_router")
+    return chosen, weight
+
+
+def moe_route_chosen(chosen: torch.Tensor, experts: int, real: int, tile_rows: int = MOE_TILE_ROWS):
+    """As ``moe_route`` for pairs whose experts a router chose (``chosen`` int32 [T, top]); experts ``real`` .. experts - 1
+    have no matrices, and a pair that names one gets no slot (pair_slot = -1)."""
+    _gpu(chosen)
+    _need(chosen.dtype == torch.int32 and chosen.dim() == 2 and chosen.is_contiguous(), "moe_route_chosen: chosen is contiguous int32 [T, top]")
+    T, top = chosen.shape
+    _need(0 <= real <= experts <= MOE_MAX_EXPERTS and experts > 0, f"moe_route_chosen: up to {MOE_MAX_EXPERTS} experts")
+    _need(tile_rows in (32, 64, 128), "moe_route_chosen: tiles of 32, 64 or 128 rows")
+    P = T * top
+    most = moe_max_tiles(P, max(real, 1), tile_rows)
+    work = torch.empty(2 * P + 3 * most + 1, dtype=torch.int32, device=chosen.device)
+    slot_pair, pair_slot, tiles, n_tiles = work[:P], work[P:2 * P], work[2 * P:2 * P + 3 * most].view(most, 3), work[2 * P + 3 * most:]
+    _check(library().tm_moe_route_chosen(None, _p(chosen), c_int(T), c_int(top), c_int(experts), c_int(real), c_int(tile_rows),
+                                         _p(slot_pair), _p(pair_slot), _p(tiles), _p(n_tiles), _stream()), "moe_route_chosen")
+    return slot_pair, pair_slot, tiles, n_tiles, tile_rows
+
+
+def moe_experts_weighted(x: torch.Tensor, routed, weight: torch.Tensor, w_up: torch.Tensor | None, w_down: torch.Tensor | None, top: int,
+                         out: torch.Tensor, shared: torch.Tensor | None = None, shared_gate: torch.Tensor | None = None) -> torch.Tensor:
+    """out[t] = sum over the token's ``top`` pairs of weight[t, k] * (Wd[e] relu(Wu[e] x[t])^2, or x[t] itself for a pair
+    without a slot) + sigmoid(shared_gate[t]) * shared[t]. w_up [E, F, K], w_down [E, N, F] (both None: every expert stands
+    for the input); ``routed`` from ``moe_route_chosen``; shared float32 [T, N] or None; shared_gate a float32 view [T, >= 1]."""
+    slot_pair, pair_slot, tiles, n_tiles, tile_rows = routed
+    _gpu(x, w_up, w_down, out, weight, shared, shared_gate)
+    T, K = x.shape
+    P = T * top
+    N = out.shape[1]
+    _need(x.stride(1) == 1 and N == K and tuple(out.shape) == (T, N) and out.is_contiguous() and x.dtype == out.dtype,
+          "moe_experts_weighted: x [T, K], out contiguous [T, K], one type")
+    _need(weight.dtype == torch.float32 and tuple(weight.shape) == (T, top) and weight.is_contiguous(), "moe_experts_weighted: weight is float32 [T, top]")
+    _need(slot_pair.numel() == P and pair_slot.numel() == P, "moe_experts_weighted: the routing belongs to another step")
+    if shared is not None:
+        _need(shared.dtype == torch.float32 and tuple(shared.shape) == (T, N) and shared.is_contiguous(), "moe_experts_weighted: shared is float32 [T, N]")
+    ldg = 0
+    if shared_gate is not None:
+        _need(shared is not None and shared_gate.dtype == torch.float32 and shared_gate.dim() == 2 and shared_gate.shape[0] == T
+              and shared_gate.stride(1) == 1, "moe_experts_weighted: shared_gate is a float32 view [T, >= 1] beside a shared result")
+        ldg = shared_gate.stride(0) if T > 1 else max(shared_gate.stride(0), 1)
+    lib, dt = library(), c_int(code(x.dtype))
+    ldx = x.stride(0) if T > 1 else max(x.stride(0), K)
+    most = tiles.shape[0]
+    part = torch.empty((max(P, 1), N), dtype=torch.float32, device=x.device)
+    if w_up is not None and most > 0:
+        E, F, K2 = w_up.shape
+        _need(K2 == K and tuple(w_down.shape) == (E, N, F) and w_up.is_contiguous() and w_down.is_contiguous()
+              and x.dtype == w_up.dtype == w_down.dtype, "moe_experts_weighted: w_up [E, F, K], w_down [E, N, F], one type")
+        act = torch.empty((P, F), dtype=x.dtype, device=x.device)
+        if x.dtype == torch.bfloat16 and lib.tm_moe_mfma_takes(_p(x), c_int(ldx), _p(w_up), _p(w_down), _p(act), c_int(K), c_int(F)):
+            _check(lib.tm_moe_up_act_mfma(_p(x), c_int(ldx), _p(slot_pair), c_int(top), _p(w_up), _p(act), _p(tiles), _p(n_tiles),
+                                          c_int(most), c_int(tile_rows), c_int(K), c_int(F), _stream()), "moe_up_act_mfma")
+            _check(lib.tm_moe_down_mfma(_p(act), _p(w_down), _p(part), _p(tiles), _p(n_tiles), c_int(most), c_int(tile_rows), c_int(F),
+                                        c_int(N), _stream()), "moe_down_mfma")
+        else:
+            _need(tile_rows == MOE_TILE_ROWS, "moe_experts_weighted: these products take tiles of 32 rows")
+            _check(lib.tm_moe_up_act(_p(x), c_int(ldx), _p(slot_pair), c_int(top), _p(w_up), _p(act), _p(tiles), _p(n_tiles), c_int(most),
+                                     c_int(K), c_int(F), dt, _stream()), "moe_up_act")
+            _check(lib.tm_moe_down(_p(act), _p(w_down), _p(part), _p(tiles), _p(n_tiles), c_int(most), c_int(F), c_int(N), dt, _stream()),
+                   "moe_down")
+    _check(lib.tm_moe_combine_weighted(_p(part), _p(pair_slot), _p(weight), _p(x), c_int(ldx), _p(shared), _p(shared_gate), c_int(ldg),
+                                       _p(out), c_int(T), c_int(top), c_int(N), dt, _stream()), "moe_combine_weighted")
     return out

@@ -74,26 +74,41 @@ class SandwichBlock(Block):
 
     def __init__(self, norm_in: Norm, mixer: Mixer, norm_mixed: Norm, norm_post: Norm | None = None,
                  ffn: FeedForward | None = None, norm_fed: Norm | None = None,
-                 names: tuple[str, str, str, str, str, str] = ("norm1", "mix.", "norm1b", "norm2", "mlp.", "norm2b")):
+                 names: tuple[str, str, str, str, str, str] = ("norm1", "mix.", "norm1b", "norm2", "mlp.", "norm2b"),
+                 scales: tuple[str, str] | None = None):
+        """A norm in front may be a ``PassThrough`` (the sublayer reads the stream itself). ``scales``: names, under the
+        layer's prefix, of per-channel vectors that multiply the two normed results (a layer scale); they are folded into
+        the weights of the norms behind the sublayers when the tensors are loaded."""
         if (ffn is None) != (norm_post is None) or (ffn is None) != (norm_fed is None):
             raise ValueError("a feed-forward comes with the norm before it and the norm behind it, or not at all")
         self.norm_in, self.mixer, self.norm_mixed = norm_in, mixer, norm_mixed
         self.norm_post, self.ffn, self.norm_fed = norm_post, ffn, norm_fed
         self.names = names
+        self.scales = scales
 
     def _parts(self):
         return [(p, n) for p, n in zip((self.norm_in, self.mixer, self.norm_mixed, self.norm_post, self.ffn, self.norm_fed),
                                        self.names) if p is not None]
 
+    def _scaled(self):
+        if self.scales is None:
+            return []
+        return [(n, name) for n, name in zip((self.norm_mixed, self.norm_fed), self.scales) if n is not None]
+
     def tensor_specs(self, prefix: str):
+        from tokenmill_amd.weights.loader import TensorSpec
         specs = {}
         for part, name in self._parts():
             specs.update(part.tensor_specs(prefix + name))
+        for norm, name in self._scaled():
+            specs[prefix + name] = TensorSpec((norm.hidden,), init="ones")
         return specs
 
     def load(self, tensors, prefix: str) -> None:
         for part, name in self._parts():
             part.load(tensors, prefix + name)
+        for norm, name in self._scaled():
+            norm.fold(tensors[prefix + name])
 
     def prepare(self, pack_weights: bool) -> None:
         for part, _ in self._parts():

@@ -44,17 +44,26 @@ class GroupRMSNorm(Norm):
     the next sublayer's input while such a result is pending does both in one kernel when the two agree on
     groups and eps."""
 
-    def __init__(self, hidden: int, eps: float, groups: int = 1, name: str = "weight"):
+    def __init__(self, hidden: int, eps: float, groups: int = 1, name: str = "weight", one_plus: bool = False):
+        """``one_plus``: the checkpoint stores the weight around zero and the norm multiplies by 1 + w; the sum is made
+        once, at load, in 32-bit."""
         if groups < 1 or hidden % groups:
             raise ValueError(f"{groups} groups do not divide a width of {hidden}")
-        self.hidden, self.eps, self.groups, self.name = hidden, float(eps), groups, name
+        self.hidden, self.eps, self.groups, self.name, self.one_plus = hidden, float(eps), groups, name, one_plus
         self.weight: torch.Tensor | None = None
 
     def tensor_specs(self, prefix: str):
-        return {f"{prefix}{self.name}": TensorSpec((self.hidden,), init="ones")}
+        return {f"{prefix}{self.name}": TensorSpec((self.hidden,), init="normal" if self.one_plus else "ones")}
 
     def load(self, tensors, prefix: str) -> None:
         self.weight = tensors[f"{prefix}{self.name}"]
+        if self.one_plus:
+            self.weight = (1.0 + self.weight.float()).contiguous()
+
+    def fold(self, scale: torch.Tensor) -> None:
+        """Multiply a per-channel scale that follows the norm (a layer scale) into its weight, in 32-bit: one vector where
+        the model has two."""
+        self.weight = (self.weight.float() * scale.float()).contiguous()
 
     def _cost(self, n: int, out_bytes: int, added: int):
         return n * self.hidden * (4 + out_bytes + added), 0
@@ -81,6 +90,35 @@ class GroupRMSNorm(Norm):
     def add_normed(self, resid, y) -> None:
         with profiling.label("norm", lambda: self._cost(resid.shape[0], 4, y.element_size())):
             ops.group_norm(resid, y, self.weight, None, None, self.groups, self.eps)
+
+
+class PassThrough(Norm):
+    """No norm in front of a sublayer: its input is the residual stream itself, rounded to the model's type. What is still
+    pending on the stream (a sublayer's result and the norm it has to pass) is added by the same kernel."""
+
+    def __init__(self, hidden: int):
+        self.hidden = hidden
+
+    def add_norm(self, resid, delta, out_dtype, rows=None, delta_norm: Norm | None = None):
+        n = resid.shape[0] if rows is None else rows.numel()
+        out = torch.empty((n, self.hidden), dtype=out_dtype, device=resid.device)
+        post, groups, eps = None, 1, 1.0
+        if delta is not None and delta_norm is not None:
+            if isinstance(delta_norm, GroupRMSNorm):
+                post, groups, eps = delta_norm.weight, delta_norm.groups, delta_norm.eps
+            elif rows is None:
+                delta_norm.add_normed(resid, delta)
+                delta = None
+            else:
+                resid = resid.index_select(0, rows.long())
+                delta_norm.add_normed(resid, delta.index_select(0, rows.long()))
+                delta, rows = None, None
+        added = 0 if delta is None else (4 if rows is None else 0) + delta.element_size()
+        with profiling.label("norm", lambda: (n * self.hidden * (4 + out.element_size() + added), 0)):
+            return ops.group_norm(resid, delta, post, None, out, groups, eps, rows)
+
+    def add_normed(self, resid, y) -> None:
+        raise NotImplementedError("a pass-through stands in front of a sublayer, not behind it")
 
 
 class GatedAdd:

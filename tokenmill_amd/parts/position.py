@@ -6,6 +6,8 @@ the kernel that also stores k and v into the cache.
 """
 from __future__ import annotations
 
+import math
+
 import torch
 
 from tokenmill_amd.hip import ops
@@ -18,9 +20,23 @@ class RotaryEmbedding(PositionEncoding):
     with kernels of its own (the kernel library's attention operation knows the first pairing only)."""
 
     def __init__(self, head_dim: int, theta: float, max_positions: int, rotary_dim: int | None = None,
-                 interleaved: bool = False):
+                 interleaved: bool = False, scaling: dict | None = None, exact: bool = False):
+        """``scaling`` (factor, original, fast, slow): the frequencies of pairs that turn fewer than ``slow`` times over
+        ``original`` positions are divided by ``factor``, those that turn more than ``fast`` times stay, and the pairs between
+        are blended linearly over the pair index; cos and sin are multiplied by 0.1 ln(factor) + 1. With j(t) =
+        rotary_dim * ln(original / (2 pi t)) / (2 ln theta): lo = max(floor(j(fast)), 0), hi = min(ceil(j(slow)),
+        rotary_dim - 1), ramp_i = clamp((i - lo) / max(hi - lo, 0.001), 0, 1), f_i <- f_i / factor * ramp_i + f_i (1 - ramp_i).
+        ``exact``: the frequencies are computed in 64-bit and rounded once to 32-bit (always so with ``scaling``)."""
         self.head_dim = head_dim
         self.interleaved = interleaved
+        self.scaling = dict(scaling) if scaling else None
+        self.exact = exact or self.scaling is not None
+        if self.scaling is not None:
+            for key in ("factor", "original", "fast", "slow"):
+                if key not in self.scaling:
+                    raise ValueError(f"rotary scaling has no '{key}'")
+            if not float(self.scaling["factor"]) > 0:
+                raise ValueError("the rotary scaling factor must be positive")
         self.rotary_dim = rotary_dim or head_dim
         if self.rotary_dim % 2 or self.rotary_dim > head_dim:
             raise ValueError(f"rotary_dim {self.rotary_dim} must be even and at most head_dim {head_dim}")
@@ -29,12 +45,35 @@ class RotaryEmbedding(PositionEncoding):
         self.cos: torch.Tensor | None = None
         self.sin: torch.Tensor | None = None
 
-    def build_tables(self, device) -> None:
+    def frequencies(self) -> tuple[torch.Tensor, float]:
+        """(float32 [rotary_dim / 2] angle per position of every pair, what cos and sin are multiplied by)."""
         d = self.rotary_dim
-        inv_freq = 1.0 / (self.theta ** (torch.arange(0, d, 2, dtype=torch.int64).float() / d))
-        freqs = torch.outer(torch.arange(self.max_positions).float(), inv_freq)     # [max_pos, d/2]
-        self.cos = freqs.cos().contiguous().to(device)
-        self.sin = freqs.sin().contiguous().to(device)
+        if not self.exact:
+            return 1.0 / (self.theta ** (torch.arange(0, d, 2, dtype=torch.int64).float() / d)), 1.0
+        i = torch.arange(d // 2, dtype=torch.float64)
+        f = self.theta ** (-2.0 * i / d)
+        sc = self.scaling
+        if sc is None:
+            return f.float(), 1.0
+        factor, original = float(sc["factor"]), float(sc["original"])
+
+        def pair_of(turns: float) -> float:
+            return d * math.log(original / (2.0 * math.pi * turns)) / (2.0 * math.log(self.theta))
+
+        lo = max(math.floor(pair_of(float(sc["fast"]))), 0)
+        hi = min(math.ceil(pair_of(float(sc["slow"]))), d - 1)
+        ramp = ((i - lo) / max(hi - lo, 0.001)).clamp(0.0, 1.0)
+        f = f / factor * ramp + f * (1.0 - ramp)
+        return f.float(), 0.1 * math.log(factor) + 1.0
+
+    def build_tables(self, device) -> None:
+        inv_freq, magnitude = self.frequencies()
+        freqs = torch.outer(torch.arange(self.max_positions).float(), inv_freq)     # [max_pos, d/2], 32-bit angles
+        cos, sin = freqs.cos(), freqs.sin()
+        if magnitude != 1.0:
+            cos, sin = cos * magnitude, sin * magnitude
+        self.cos = cos.contiguous().to(device)
+        self.sin = sin.contiguous().to(device)
 
     def load(self, tensors, prefix: str) -> None:
         device = next(iter(tensors.values())).device

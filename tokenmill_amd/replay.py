@@ -44,7 +44,7 @@ class ReplaySession:
         # --max-tokens bounds what all live requests hold together; one request can be no longer than that,
         # nor than the model's own position tables reach
         _, model_config = load_config(model_dir)
-        max_positions = min(max_tokens, getattr(model_config, "max_position_embeddings", max_tokens))
+        max_positions = min(max_tokens, getattr(model_config, "max_position_embeddings", None) or max_tokens)
         self.model = load_model(model_dir, dtype, device, max_positions=max_positions)
         self.page_size = page_size
         # every request's tokens count rounded up to ROUND_TO; a page that does not divide that may leave
