@@ -48,6 +48,21 @@ int tm_attn_paged_generic_ext(const void* q, int q_stride, void* out, int out_st
                               int KVH, int D, int DV, int page, float scale, int window, float softcap, const float* gate, int ldg,
                               int dtype, hipStream_t stream);
 
+// The matrix-unit attention kernels with capped scores (softcap > 0: s <- softcap * tanh(s / softcap); 0: as the plain entries).
+int tm_attn_prefill_mfma_cap(const void* q, int q_stride, void* out, int out_stride, const void* k_pool, const void* v_pool,
+                             const int* block_tables, int table_width, const int* tiles, int n_tiles, int H, int KVH, int D, int page,
+                             float scale, int window, float softcap, hipStream_t stream);
+int tm_attn_prefill_shared_cap(const void* q, int q_stride, void* out, int out_stride, const void* k_pool, const void* v_pool,
+                               const int* block_tables, int table_width, const int* tiles, int n_tiles, int H, int KVH, int D, int page,
+                               float scale, int window, float softcap, hipStream_t stream);
+int tm_attn_prefill_f32_cap(const void* q, int q_stride, void* out, int out_stride, const void* k_pool, const void* v_pool,
+                            const int* block_tables, int table_width, const int* tiles, int n_tiles, int H, int KVH, int D, int page,
+                            float scale, int window, float softcap, hipStream_t stream);
+int tm_attn_decode_mfma_cap(const void* q, int q_stride, void* out, int out_stride, const void* k_pool, const void* v_pool,
+                            const int* block_tables, int table_width, const int* context_lens, float* part_o, float* part_ml,
+                            int max_chunks, int S, int H, int KVH, int D, int page, float scale, int window, float softcap,
+                            hipStream_t stream);
+
 // q and k normed over the whole projection, rotated and stored (attention_prepare.hip): see the head of that file.
 int tm_whole_norm_rope_store(const float* proj, int ld, void* q_out, int dtype, int T, int H, int G, int D, int Dv, int rot,
                              int interleaved, const float* q_w, const float* k_w, float eps, const float* cos_t, const float* sin_t,

@@ -124,7 +124,7 @@ __device__ __forceinline__ void load_keys64(Keys64<D>& kv, const bf16_t* __restr
 // m is in units of score * scale * log2(e).
 template <int D>
 __device__ __forceinline__ void attend_keys64(const Keys64<D>& kv, const Bf16x8Bits (&qreg)[D / 32], int wbase, int ctx,
-                                              int lo, float scale_log2, int g, float& m, float& l,
+                                              int lo, float scale_log2, float cap_in, float cap_out, int g, float& m, float& l,
                                               f32x4_t (&o)[D / 16]) {
     constexpr int NDC = D / 32, NDT = D / 16;
     float sc[4][4];                                                 // [tile][row 4g+i of the tile] for head r
@@ -137,7 +137,9 @@ __device__ __forceinline__ void attend_keys64(const Keys64<D>& kv, const Bf16x8B
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             const int kj = wbase + tile_key(t, 4 * g + i);
-            sc[t][i] = (kj < ctx && kj >= lo) ? acc[i] * scale_log2 : -INFINITY;
+            // cap_in > 0: capped scores, cap * tanh(score * scale / cap), in units of log2 like the plain ones
+            const float sv = cap_in > 0.f ? cap_out * tanh_fast(acc[i] * cap_in) : acc[i] * scale_log2;
+            sc[t][i] = (kj < ctx && kj >= lo) ? sv : -INFINITY;
         }
     }
     m = -INFINITY;
@@ -189,13 +191,13 @@ template <int D>
 __device__ __forceinline__ void wave_keys64(const Bf16x8Bits (&qreg)[D / 32], const bf16_t* __restrict__ k_pool,
                                             const bf16_t* __restrict__ v_pool, const int* __restrict__ table,
                                             int table_width, int wbase, int ctx, int lo, int kvh, int KVH,
-                                            int page_shift, float scale_log2, int r, int g, float& m, float& l,
+                                            int page_shift, float scale_log2, float cap_in, float cap_out, int r, int g, float& m, float& l,
                                             f32x4_t (&o)[D / 16]) {
     int entry[4];
     load_table_entries(entry, table, table_width, wbase, page_shift);
     Keys64<D> kv;
     load_keys64<D>(kv, k_pool, v_pool, entry, wbase, ctx, lo, kvh, KVH, page_shift, r, g);
-    attend_keys64<D>(kv, qreg, wbase, ctx, lo, scale_log2, g, m, l, o);
+    attend_keys64<D>(kv, qreg, wbase, ctx, lo, scale_log2, cap_in, cap_out, g, m, l, o);
 }
 
 template <int D>
@@ -218,7 +220,7 @@ template <int D, int WAVES>
 __global__ __launch_bounds__(64 * WAVES) void attn_decode_block_kernel(
     const bf16_t* __restrict__ q, int q_stride, bf16_t* __restrict__ out, int out_stride,
     const bf16_t* __restrict__ k_pool, const bf16_t* __restrict__ v_pool, const int* __restrict__ block_tables,
-    int table_width, const int* __restrict__ context_lens, int H, int KVH, int page_shift, float scale_log2,
+    int table_width, const int* __restrict__ context_lens, int H, int KVH, int page_shift, float scale_log2, float cap_in, float cap_out,
     int window) {
     constexpr int NDT = D / 16;
     __shared__ float s_m[WAVES][16], s_l[WAVES][16];
@@ -254,7 +256,7 @@ __global__ __launch_bounds__(64 * WAVES) void attn_decode_block_kernel(
     for (int wbase = first + wave * AD_WKEYS; wbase < ctx; wbase += WAVES * AD_WKEYS) {
         float mi, li;
         f32x4_t oi[NDT];
-        wave_keys64<D>(qreg, k_pool, v_pool, table, table_width, wbase, ctx, lo, kvh, KVH, page_shift, scale_log2, r, g, mi, li, oi);
+        wave_keys64<D>(qreg, k_pool, v_pool, table, table_width, wbase, ctx, lo, kvh, KVH, page_shift, scale_log2, cap_in, cap_out, r, g, mi, li, oi);
         fold(mi, li, oi);
     }
     // merge the wavefronts in wavefront order; lane: head r, d = 16 dt + 4 g + i
@@ -311,7 +313,7 @@ __global__ __launch_bounds__(256) void attn_decode_split_kernel(
     const bf16_t* __restrict__ q, int q_stride, const bf16_t* __restrict__ k_pool,
     const bf16_t* __restrict__ v_pool, const int* __restrict__ block_tables, int table_width,
     const int* __restrict__ context_lens, float* __restrict__ part_o, float* __restrict__ part_ml,
-    int max_chunks, int H, int KVH, int page_shift, float scale_log2, int window) {
+    int max_chunks, int H, int KVH, int page_shift, float scale_log2, float cap_in, float cap_out, int window) {
     constexpr int NDT = D / 16;
     __shared__ float s_m[4][16], s_l[4][16];
     __shared__ float s_o[4][16][D + 1];
@@ -335,7 +337,7 @@ __global__ __launch_bounds__(256) void attn_decode_split_kernel(
     {
         Keys64<D> kv;
         load_keys64<D>(kv, k_pool, v_pool, entry, wbase, ctx, lo, kvh, KVH, page_shift, r, g);
-        attend_keys64<D>(kv, qreg, wbase, ctx, lo, scale_log2, g, m, l, o);
+        attend_keys64<D>(kv, qreg, wbase, ctx, lo, scale_log2, cap_in, cap_out, g, m, l, o);
     }
     if (g == 0) {
         s_m[wave][r] = m;
@@ -498,10 +500,11 @@ template <int D>
 static int launch_decode(const void* q, int q_stride, void* out, int out_stride, const void* k_pool,
                          const void* v_pool, const int* block_tables, int table_width, const int* context_lens,
                          float* part_o, float* part_ml, int max_chunks, int S, int H, int KVH, int page,
-                         float scale, int window, hipStream_t stream) {
+                         float scale, int window, float softcap, hipStream_t stream) {
     int page_shift = 0;
     while ((1 << page_shift) < page) ++page_shift;
     const float scale_log2 = scale * 1.4426950408889634f;
+    const float cap_in = softcap > 0.f ? scale / softcap : 0.f, cap_out = softcap * 1.4426950408889634f;
     constexpr int WAVES = D <= 32 ? 16 : 8;       // 16 wavefronts leave 128 registers each: enough for D = 32 only
     // few (request, kv head) pairs: more blocks than pairs are needed to pull the cache at speed; the caller
     // asks for that by bringing the scratch memory
@@ -509,13 +512,13 @@ static int launch_decode(const void* q, int q_stride, void* out, int out_stride,
     if (!split) {
         attn_decode_block_kernel<D, WAVES><<<dim3(S, KVH), 64 * WAVES, 0, stream>>>(
             (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, (const bf16_t*)k_pool, (const bf16_t*)v_pool,
-            block_tables, table_width, context_lens, H, KVH, page_shift, scale_log2, window);
+            block_tables, table_width, context_lens, H, KVH, page_shift, scale_log2, cap_in, cap_out, window);
         TM_CHECK_LAUNCH();
         return TM_OK;
     }
     attn_decode_split_kernel<D><<<dim3(S, KVH, max_chunks), 256, 0, stream>>>(
         (const bf16_t*)q, q_stride, (const bf16_t*)k_pool, (const bf16_t*)v_pool, block_tables, table_width,
-        context_lens, part_o, part_ml, max_chunks, H, KVH, page_shift, scale_log2, window);
+        context_lens, part_o, part_ml, max_chunks, H, KVH, page_shift, scale_log2, cap_in, cap_out, window);
     TM_CHECK_LAUNCH();
     if (max_chunks <= TM_WAVE)
         attn_decode_merge_kernel<<<dim3(S, H), 64 * AD_MERGE_WAVES, 0, stream>>>(
@@ -531,11 +534,13 @@ static int launch_decode(const void* q, int q_stride, void* out, int out_stride,
 // context_lens: first decode request. part_o: float [S, H, max_chunks, D] and part_ml: [S, H, max_chunks, 2]
 // are scratch for the split kernels, which run when both are given (the caller gives them when the
 // (request, kv head) pairs alone are too few blocks for the chip); without them the block kernel runs.
-extern "C" int tm_attn_decode_mfma(const void* q, int q_stride, void* out, int out_stride, const void* k_pool,
-                                   const void* v_pool, const int* block_tables, int table_width,
-                                   const int* context_lens, float* part_o, float* part_ml, int max_chunks, int S,
-                                   int H, int KVH, int D, int page, float scale, int window, hipStream_t stream) {
+// softcap > 0: a score s (scaled) becomes softcap * tanh(s / softcap) before the softmax.
+extern "C" int tm_attn_decode_mfma_cap(const void* q, int q_stride, void* out, int out_stride, const void* k_pool,
+                                       const void* v_pool, const int* block_tables, int table_width,
+                                       const int* context_lens, float* part_o, float* part_ml, int max_chunks, int S,
+                                       int H, int KVH, int D, int page, float scale, int window, float softcap, hipStream_t stream) {
     if (S <= 0) return TM_OK;
+    if (!(softcap >= 0.f)) return TM_ERR_ARG;
     if (H <= 0 || KVH <= 0 || H % KVH || H / KVH > 16 || page < 16 || (page & (page - 1)) || max_chunks <= 0 ||
         !(scale > 0.f) || max_chunks > 65535 || KVH > 65535 || window < 0 || table_width <= 0 || (q_stride % 8) ||
         ((uintptr_t)q % 16) || (out_stride % 4) || ((uintptr_t)out % 8) || q_stride < H * D || out_stride < H * D)
@@ -543,7 +548,7 @@ extern "C" int tm_attn_decode_mfma(const void* q, int q_stride, void* out, int o
 #define TM_DECODE_CASE(DD)                                                                                        \
     case DD:                                                                                                      \
         return launch_decode<DD>(q, q_stride, out, out_stride, k_pool, v_pool, block_tables, table_width,         \
-                                 context_lens, part_o, part_ml, max_chunks, S, H, KVH, page, scale, window, stream)
+                                 context_lens, part_o, part_ml, max_chunks, S, H, KVH, page, scale, window, softcap, stream)
     switch (D) {
         TM_DECODE_CASE(32);
         TM_DECODE_CASE(64);
@@ -553,4 +558,12 @@ extern "C" int tm_attn_decode_mfma(const void* q, int q_stride, void* out, int o
             return TM_ERR_ARG;
     }
 #undef TM_DECODE_CASE
+}
+
+extern "C" int tm_attn_decode_mfma(const void* q, int q_stride, void* out, int out_stride, const void* k_pool,
+                                   const void* v_pool, const int* block_tables, int table_width,
+                                   const int* context_lens, float* part_o, float* part_ml, int max_chunks, int S,
+                                   int H, int KVH, int D, int page, float scale, int window, hipStream_t stream) {
+    return tm_attn_decode_mfma_cap(q, q_stride, out, out_stride, k_pool, v_pool, block_tables, table_width, context_lens, part_o, part_ml,
+                                   max_chunks, S, H, KVH, D, page, scale, window, 0.f, stream);
 }

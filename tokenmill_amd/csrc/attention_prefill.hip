@@ -77,7 +77,7 @@ __device__ __forceinline__ void load_kv_block(KVBlock<D>& blk, int2 pages, int s
 // One block of 32 keys against the wavefront's heads.
 template <int D, int HPW>
 __device__ __forceinline__ void attend_block(KVBlock<D>& blk, HeadState<D, HPW>& st, const PFrag (&qf)[HPW][D / 32],
-                                             int key0, int nh, const TileView& tv, int g, float scale_log2) {
+                                             int key0, int nh, const TileView& tv, int g, float scale_log2, float cap_in, float cap_out) {
     constexpr int NDC = D / 32, NDT = D / 16;
     // values of keys nobody may see (beyond the newest key) can hold anything: clear them
     if (key0 + 31 > tv.last_key) {
@@ -107,6 +107,11 @@ __device__ __forceinline__ void attend_block(KVBlock<D>& blk, HeadState<D, HPW>&
 #pragma unroll
             for (int c = 0; c < NDC; ++c)
                 acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(blk.k[t][c].b, qf[hh][c].b, acc, 0, 0, 0);
+            // capped scores: cap * tanh(score * scale / cap), kept in units of 1 / scale like the plain ones
+            if (cap_in > 0.f) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) acc[i] = cap_out * tanh_fast(acc[i] * cap_in);
+            }
             sc[hh][t] = acc;
         }
     }
@@ -183,7 +188,7 @@ __global__ __launch_bounds__(64 * KS) void attn_prefill_mfma_kernel(
     const bf16_t* __restrict__ q, int q_stride, bf16_t* __restrict__ out, int out_stride,
     const bf16_t* __restrict__ k_pool, const bf16_t* __restrict__ v_pool, const int* __restrict__ block_tables,
     int table_width, const int* __restrict__ tiles, int n_tiles, int pair, int H, int KVH, int page_shift,
-    float scale_log2, int window) {
+    float scale_log2, float cap_in, float cap_out, int window) {
     constexpr int NDC = D / 32, NDT = D / 16;
     __shared__ float s_m[KS][16], s_l[KS][16];
     __shared__ float s_o[KS][16][D + 1];
@@ -249,7 +254,7 @@ __global__ __launch_bounds__(64 * KS) void attn_prefill_mfma_kernel(
                 slot = -1;
             }
             load_kv_block<D>(bb, pages, slot + 1, k_pool, v_pool, kvh, KVH, page_shift, off);
-            attend_block<D, HPW>(ba, st, qf, kb * 32, nh, tv, g, scale_log2);
+            attend_block<D, HPW>(ba, st, qf, kb * 32, nh, tv, g, scale_log2, cap_in, cap_out);
             kb += KS;
             ++slot;
             if (kb > kb1) break;
@@ -258,7 +263,7 @@ __global__ __launch_bounds__(64 * KS) void attn_prefill_mfma_kernel(
                 slot = -1;
             }
             load_kv_block<D>(ba, pages, slot + 1, k_pool, v_pool, kvh, KVH, page_shift, off);
-            attend_block<D, HPW>(bb, st, qf, kb * 32, nh, tv, g, scale_log2);
+            attend_block<D, HPW>(bb, st, qf, kb * 32, nh, tv, g, scale_log2, cap_in, cap_out);
             kb += KS;
             ++slot;
         }
@@ -310,7 +315,7 @@ template <int D> struct PrefillShape { static constexpr int HPW = D <= 64 ? 4 : 
 template <int D, int HPW>
 static void launch_split_keys(const void* q, int q_stride, void* out, int out_stride, const void* k_pool, const void* v_pool,
                               const int* block_tables, int table_width, const int* tiles, int n_tiles, int H, int KVH,
-                              int page_shift, float scale_log2, int window, hipStream_t stream) {
+                              int page_shift, float scale_log2, float cap_in, float cap_out, int window, hipStream_t stream) {
     constexpr int KS = PrefillShape<D>::KS;
     const int splits = (H / KVH + HPW - 1) / HPW;
     // fold the table in two once the folded launch still gives every CU a block
@@ -318,14 +323,17 @@ static void launch_split_keys(const void* q, int q_stride, void* out, int out_st
     dim3 grid(pair ? (n_tiles + 1) / 2 : n_tiles, KVH * splits);
     attn_prefill_mfma_kernel<D, HPW, KS><<<grid, 64 * KS, 0, stream>>>(
         (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, (const bf16_t*)k_pool, (const bf16_t*)v_pool, block_tables,
-        table_width, tiles, n_tiles, pair, H, KVH, page_shift, scale_log2, window);
+        table_width, tiles, n_tiles, pair, H, KVH, page_shift, scale_log2, cap_in, cap_out, window);
 }
 
-extern "C" int tm_attn_prefill_mfma(const void* q, int q_stride, void* out, int out_stride, const void* k_pool,
-                                    const void* v_pool, const int* block_tables, int table_width, const int* tiles,
-                                    int n_tiles, int H, int KVH, int D, int page, float scale, int window,
-                                    hipStream_t stream) {
+// softcap > 0: a score s (scaled) becomes softcap * tanh(s / softcap) before the softmax
+extern "C" int tm_attn_prefill_mfma_cap(const void* q, int q_stride, void* out, int out_stride, const void* k_pool,
+                                        const void* v_pool, const int* block_tables, int table_width, const int* tiles,
+                                        int n_tiles, int H, int KVH, int D, int page, float scale, int window, float softcap,
+                                        hipStream_t stream) {
     if (n_tiles <= 0) return TM_OK;
+    if (!(softcap >= 0.f)) return TM_ERR_ARG;
+    const float cap_in = softcap > 0.f ? scale / softcap : 0.f, cap_out = softcap > 0.f ? softcap / scale : 0.f;
     if (H <= 0 || KVH <= 0 || H % KVH || page < 16 || (page & (page - 1)) || window < 0 || table_width <= 0 ||
         (q_stride % 8) || ((uintptr_t)q % 16) || (out_stride % 2) || ((uintptr_t)out % 4) || q_stride < H * D ||
         out_stride < H * D || !(scale > 0.f))
@@ -336,7 +344,7 @@ extern "C" int tm_attn_prefill_mfma(const void* q, int q_stride, void* out, int 
     const float scale_log2 = scale * 1.4426950408889634f;
     if ((long long)KVH * ((G + 1) / 2) > 65535) return TM_ERR_ARG;
 #define TM_SPLIT_ARGS q, q_stride, out, out_stride, k_pool, v_pool, block_tables, table_width, tiles, n_tiles, H, KVH, \
-                      page_shift, scale_log2, window, stream
+                      page_shift, scale_log2, cap_in, cap_out, window, stream
 #define TM_PREFILL_CASE(DD)                                                                                       \
     case DD: {                                                                                                    \
         constexpr int HPW = PrefillShape<DD>::HPW;                                                                \
@@ -358,4 +366,12 @@ extern "C" int tm_attn_prefill_mfma(const void* q, int q_stride, void* out, int 
 #undef TM_SPLIT_ARGS
     TM_CHECK_LAUNCH();
     return TM_OK;
+}
+
+extern "C" int tm_attn_prefill_mfma(const void* q, int q_stride, void* out, int out_stride, const void* k_pool,
+                                    const void* v_pool, const int* block_tables, int table_width, const int* tiles,
+                                    int n_tiles, int H, int KVH, int D, int page, float scale, int window,
+                                    hipStream_t stream) {
+    return tm_attn_prefill_mfma_cap(q, q_stride, out, out_stride, k_pool, v_pool, block_tables, table_width, tiles, n_tiles, H, KVH, D,
+                                    page, scale, window, 0.f, stream);
 }

@@ -30,7 +30,7 @@ template <int D>
 __global__ __launch_bounds__(64 * AF_SPLIT) void attn_prefill_f32_kernel(
     const float* __restrict__ q, int q_stride, float* __restrict__ out, int out_stride,
     const float* __restrict__ k_pool, const float* __restrict__ v_pool, const int* __restrict__ block_tables,
-    int table_width, const int* __restrict__ tiles, int H, int KVH, int page_shift, float scale, int window) {
+    int table_width, const int* __restrict__ tiles, int H, int KVH, int page_shift, float scale, int window, float softcap) {
     constexpr int DQ = D / 4;           // values of a key (or query) a lane holds
     constexpr int NDT = D / 16;         // 16-row tiles of d
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / TM_WAVE);
@@ -97,6 +97,7 @@ __global__ __launch_bounds__(64 * AF_SPLIT) void attn_prefill_f32_kernel(
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             sc[i] *= scale;
+            if (softcap > 0.f) sc[i] = softcap * tanhf(sc[i] / softcap);
             if (edge) {
                 const int kj = key0 + 4 * g + i;
                 if (kj > my_pos || kj < my_lo) sc[i] = -INFINITY;
@@ -170,11 +171,13 @@ __global__ __launch_bounds__(64 * AF_SPLIT) void attn_prefill_f32_kernel(
 // q float32 [T, >= H*D] rows, out float32 [T, >= H*D]; pools float32, K [pages, page, KVH, D], V [pages, KVH, D, page];
 // tiles int32 [n_tiles][4] = (request index, first row, tokens (1..16), position of the first token).
 // Needs D % 16 == 0 (at most 128), page a power of two >= 16, 16-byte aligned q, out and pools, strides % 4 == 0.
-extern "C" int tm_attn_prefill_f32(const void* q, int q_stride, void* out, int out_stride, const void* k_pool,
-                                   const void* v_pool, const int* block_tables, int table_width, const int* tiles,
-                                   int n_tiles, int H, int KVH, int D, int page, float scale, int window,
-                                   hipStream_t stream) {
+// softcap > 0: a score s (scaled) becomes softcap * tanh(s / softcap) before the softmax.
+extern "C" int tm_attn_prefill_f32_cap(const void* q, int q_stride, void* out, int out_stride, const void* k_pool,
+                                       const void* v_pool, const int* block_tables, int table_width, const int* tiles,
+                                       int n_tiles, int H, int KVH, int D, int page, float scale, int window, float softcap,
+                                       hipStream_t stream) {
     if (n_tiles <= 0) return TM_OK;
+    if (!(softcap >= 0.f)) return TM_ERR_ARG;
     if (H <= 0 || KVH <= 0 || H % KVH || page < 16 || (page & (page - 1)) || window < 0 || table_width <= 0 ||
         (q_stride % 4) || (out_stride % 4) || ((uintptr_t)q % 16) || ((uintptr_t)out % 16) || ((uintptr_t)k_pool % 16) ||
         ((uintptr_t)v_pool % 16) || q_stride < H * D || out_stride < H * D || !(scale > 0.f))
@@ -187,7 +190,7 @@ extern "C" int tm_attn_prefill_f32(const void* q, int q_stride, void* out, int o
     case DD:                                                                                                      \
         attn_prefill_f32_kernel<DD><<<grid, 64 * AF_SPLIT, 0, stream>>>(                                          \
             (const float*)q, q_stride, (float*)out, out_stride, (const float*)k_pool, (const float*)v_pool,       \
-            block_tables, table_width, tiles, H, KVH, page_shift, scale, window);                                 \
+            block_tables, table_width, tiles, H, KVH, page_shift, scale, window, softcap);                                 \
         break
     switch (D) {
         TM_PREFILL_F32_CASE(16);
@@ -204,4 +207,12 @@ extern "C" int tm_attn_prefill_f32(const void* q, int q_stride, void* out, int o
 #undef TM_PREFILL_F32_CASE
     TM_CHECK_LAUNCH();
     return TM_OK;
+}
+
+extern "C" int tm_attn_prefill_f32(const void* q, int q_stride, void* out, int out_stride, const void* k_pool,
+                                   const void* v_pool, const int* block_tables, int table_width, const int* tiles,
+                                   int n_tiles, int H, int KVH, int D, int page, float scale, int window,
+                                   hipStream_t stream) {
+    return tm_attn_prefill_f32_cap(q, q_stride, out, out_stride, k_pool, v_pool, block_tables, table_width, tiles, n_tiles, H, KVH, D,
+                                   page, scale, window, 0.f, stream);
 }

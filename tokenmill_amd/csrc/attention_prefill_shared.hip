@@ -128,7 +128,7 @@ struct StageCopy {
 template <int D, int HPW>
 __device__ __forceinline__ void attend_shared(const unsigned char* stage, int sub, HeadState<D, HPW>& st,
                                               const PFrag (&qf)[HPW][D / 32], int key0, const TileView& tv,
-                                              int r, int g, float scale_log2) {
+                                              int r, int g, float scale_log2, float cap_in, float cap_out) {
     constexpr int NDC = D / 32, NDT = D / 16;
     constexpr int KS = SharedShape<D>::K_STRIDE, VS = SharedShape<D>::V_STRIDE;
     // does any (query, key) pair of this block fall outside the causal / window limits?
@@ -149,6 +149,11 @@ __device__ __forceinline__ void attend_shared(const unsigned char* stage, int su
 #pragma unroll
             for (int c = 0; c < NDC; ++c)
                 acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[t][c].b, qf[hh][c].b, acc, 0, 0, 0);
+            // capped scores: cap * tanh(score * scale / cap), kept in units of 1 / scale like the plain ones
+            if (cap_in > 0.f) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) acc[i] = cap_out * tanh_fast(acc[i] * cap_in);
+            }
             sc[t] = acc;
         }
         if (edge) {
@@ -219,7 +224,7 @@ __global__ __launch_bounds__(64 * WAVES, SharedPlan<D>::WAVES_PER_SIMD) void att
     const bf16_t* __restrict__ q, int q_stride, bf16_t* __restrict__ out, int out_stride,
     const bf16_t* __restrict__ k_pool, const bf16_t* __restrict__ v_pool, const int* __restrict__ block_tables,
     int table_width, const int* __restrict__ tiles, int n_tiles, int pair, int H, int KVH, int page_shift,
-    float scale_log2, int window) {
+    float scale_log2, float cap_in, float cap_out, int window) {
     constexpr int NDC = D / 32, NDT = D / 16, THREADS = 64 * WAVES, STAGE = SharedShape<D>::STAGE, HPW = SharedPlan<D>::HPW;
     extern __shared__ __align__(16) unsigned char stages[];          // two stages
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / TM_WAVE);
@@ -288,7 +293,7 @@ __global__ __launch_bounds__(64 * WAVES, SharedPlan<D>::WAVES_PER_SIMD) void att
                 for (int sub = 0; sub < 2; ++sub) {
                     const int key0 = sb * PS_KEYS + 32 * sub;
                     if (key0 > tv.last_key || key0 + 31 < first_key) continue;     // block-uniform: nothing of it is visible
-                    attend_shared<D, HPW>(stages + cur * STAGE, sub, st, qf, key0, tv, r, g, scale_log2);
+                    attend_shared<D, HPW>(stages + cur * STAGE, sub, st, qf, key0, tv, r, g, scale_log2, cap_in, cap_out);
                 }
             }
             copy.store(stages + (cur ^ 1) * STAGE, tid, tv.last_key + 1 - next * PS_KEYS);
@@ -319,7 +324,7 @@ __global__ __launch_bounds__(64 * WAVES, SharedPlan<D>::WAVES_PER_SIMD) void att
 template <int D, int WAVES>
 static int launch_shared(const void* q, int q_stride, void* out, int out_stride, const void* k_pool, const void* v_pool,
                          const int* block_tables, int table_width, const int* tiles, int n_tiles, int H, int KVH,
-                         int page_shift, float scale_log2, int window, hipStream_t stream) {
+                         int page_shift, float scale_log2, float cap_in, float cap_out, int window, hipStream_t stream) {
     constexpr int lds = 2 * SharedShape<D>::STAGE;
     static bool raised = false;
     if (lds > 48 * 1024 && !raised) {
@@ -333,7 +338,7 @@ static int launch_shared(const void* q, int q_stride, void* out, int out_stride,
     dim3 grid(pair ? (n_tiles + 1) / 2 : n_tiles, KVH);
     attn_prefill_shared_kernel<D, WAVES><<<grid, 64 * WAVES, lds, stream>>>(
         (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, (const bf16_t*)k_pool, (const bf16_t*)v_pool, block_tables,
-        table_width, tiles, n_tiles, pair, H, KVH, page_shift, scale_log2, window);
+        table_width, tiles, n_tiles, pair, H, KVH, page_shift, scale_log2, cap_in, cap_out, window);
     TM_CHECK_LAUNCH();
     return TM_OK;
 }
@@ -346,11 +351,14 @@ extern "C" int tm_attn_prefill_shared_takes(int H, int KVH, int D) {
     return G <= 8 * (D <= 64 ? SharedPlan<64>::HPW : SharedPlan<128>::HPW);
 }
 
-extern "C" int tm_attn_prefill_shared(const void* q, int q_stride, void* out, int out_stride, const void* k_pool,
-                                      const void* v_pool, const int* block_tables, int table_width, const int* tiles,
-                                      int n_tiles, int H, int KVH, int D, int page, float scale, int window,
-                                      hipStream_t stream) {
+// softcap > 0: a score s (scaled) becomes softcap * tanh(s / softcap) before the softmax
+extern "C" int tm_attn_prefill_shared_cap(const void* q, int q_stride, void* out, int out_stride, const void* k_pool,
+                                          const void* v_pool, const int* block_tables, int table_width, const int* tiles,
+                                          int n_tiles, int H, int KVH, int D, int page, float scale, int window, float softcap,
+                                          hipStream_t stream) {
     if (n_tiles <= 0) return TM_OK;
+    if (!(softcap >= 0.f)) return TM_ERR_ARG;
+    const float cap_in = softcap > 0.f ? scale / softcap : 0.f, cap_out = softcap > 0.f ? softcap / scale : 0.f;
     if (!tm_attn_prefill_shared_takes(H, KVH, D) || page < 16 || (page & (page - 1)) || window < 0 || table_width <= 0 ||
         (q_stride % 8) || ((uintptr_t)q % 16) || (out_stride % 4) || ((uintptr_t)out % 8) || q_stride < H * D ||
         out_stride < H * D || !(scale > 0.f))
@@ -361,7 +369,7 @@ extern "C" int tm_attn_prefill_shared(const void* q, int q_stride, void* out, in
     while ((1 << page_shift) < page) ++page_shift;
     const float scale_log2 = scale * 1.4426950408889634f;
 #define TM_SHARED_ARGS q, q_stride, out, out_stride, k_pool, v_pool, block_tables, table_width, tiles, n_tiles, H, KVH, \
-                       page_shift, scale_log2, window, stream
+                       page_shift, scale_log2, cap_in, cap_out, window, stream
 #define TM_SHARED_CASE(DD)                                                          \
     case DD:                                                                        \
         if (need <= 2) return launch_shared<DD, 2>(TM_SHARED_ARGS);                 \
@@ -379,4 +387,12 @@ extern "C" int tm_attn_prefill_shared(const void* q, int q_stride, void* out, in
     }
 #undef TM_SHARED_CASE
 #undef TM_SHARED_ARGS
+}
+
+extern "C" int tm_attn_prefill_shared(const void* q, int q_stride, void* out, int out_stride, const void* k_pool,
+                                      const void* v_pool, const int* block_tables, int table_width, const int* tiles,
+                                      int n_tiles, int H, int KVH, int D, int page, float scale, int window,
+                                      hipStream_t stream) {
+    return tm_attn_prefill_shared_cap(q, q_stride, out, out_stride, k_pool, v_pool, block_tables, table_width, tiles, n_tiles, H, KVH,
+                                      D, page, scale, window, 0.f, stream);
 }

@@ -50,6 +50,8 @@ struct TmAttentionOp {          // resid += o(attention(rope(qkv(norm(resid)))))
     int page;
     int group;                  // which of the step's block tables and slot mappings
     int write;                  // 0: this call reads a cache that another call writes
+    float softcap;              // > 0: a scaled score s becomes softcap * tanh(s / softcap) before the softmax
+    int outside;                // 1: q always comes projected, encoded and stored (TmStream.qkv); `qkv` and `norm` are not looked at
 };
 
 struct TmFfnOp {                // resid += down(silu(gate(n)) * up(n)), n = norm(resid)
@@ -90,6 +92,9 @@ struct TmStream {
     const void* qkv;            // in: q|k|v [T, (H + 2 KVH) D] of the first operation (an attention), already projected,
                                 // position-encoded and stored in the cache (only attention and output projection run), or null
     int accumulate;             // 0: nothing is added into resid by an operation's last product: its result is left in `delta`
+    int qkv_stride;             // elements between the rows of `qkv` (0: (H + 2 KVH) D); a caller that hands in q alone says H D
+    const float* gate;          // with `qkv`: a gate per (token, head), rows `ldg` apart: head h of token t is multiplied by
+    int ldg;                    // sigmoid(gate[t * ldg + h]) between the attention and the output projection; or null
 };
 
 struct TmProgram;

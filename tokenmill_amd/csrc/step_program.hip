@@ -181,6 +181,9 @@ struct Run {
     const void* delta;                  // product output still to be added to the residual stream
     const void* x_in;                   // the next operation's input, already normed
     const void* qkv_in;                 // the next (attention) operation's q|k|v, already encoded and stored
+    int qkv_in_stride = 0;              // its row stride (0: the whole q|k|v)
+    const float* gate_in = nullptr;     // a gate per (token, head) for that operation's result
+    int gate_ld = 0;
     bool accumulate;
     // workspace
     void *x, *qkv, *attn, *gu, *act, *delta_buf, *hnorm;
@@ -280,8 +283,11 @@ struct Run {
         int rc = TM_OK;
         if (qkv_in) {                       // projected, encoded and stored by the caller
             q = qkv_in;
-            q_stride = QKV;
+            q_stride = qkv_in_stride > 0 ? qkv_in_stride : QKV;
+            if (q_stride < HD) return TM_ERR_ARG;
             qkv_in = nullptr;
+        } else if (a.outside) {
+            return TM_ERR_ARG;              // this operation has no projection of its own
         } else {
             Label l(this, op, TM_LABEL_QKV);
             const bool own_norm = x_in == nullptr;
@@ -342,18 +348,18 @@ struct Run {
                 if (tm_prefill_shares_keys(a.D, a.H, a.KVH, s->n_tiles) && tm_attn_prefill_shared_takes(a.H, a.KVH, a.D) &&
                     HD % 4 == 0 && aligned(attn, 8)) {
                     ++p->taken[TM_PREFILL_SHARED_KEYS];
-                    rc = tm_attn_prefill_shared(q, q_stride, attn, HD, a.k_pool, a.v_pool, tables, W, s->prefill_tiles,
-                                                s->n_tiles, a.H, a.KVH, a.D, a.page, a.scale, a.window, stream);
+                    rc = tm_attn_prefill_shared_cap(q, q_stride, attn, HD, a.k_pool, a.v_pool, tables, W, s->prefill_tiles,
+                                                    s->n_tiles, a.H, a.KVH, a.D, a.page, a.scale, a.window, a.softcap, stream);
                 } else {
                     ++p->taken[TM_PREFILL_SPLIT_KEYS];
-                    rc = tm_attn_prefill_mfma(q, q_stride, attn, HD, a.k_pool, a.v_pool, tables, W, s->prefill_tiles,
-                                              s->n_tiles, a.H, a.KVH, a.D, a.page, a.scale, a.window, stream);
+                    rc = tm_attn_prefill_mfma_cap(q, q_stride, attn, HD, a.k_pool, a.v_pool, tables, W, s->prefill_tiles,
+                                                  s->n_tiles, a.H, a.KVH, a.D, a.page, a.scale, a.window, a.softcap, stream);
                 }
                 done_prefill = true;
             } else if (tp && s->n_tiles > 0 && s->prefill_tiles && dtype == TM_F32 && a.D % 16 == 0 && a.D >= 16 &&
                        a.D <= 128 && page_ok && q_stride % 4 == 0 && aligned(q, 16)) {
-                rc = tm_attn_prefill_f32(q, q_stride, attn, HD, a.k_pool, a.v_pool, tables, W, s->prefill_tiles, s->n_tiles, a.H,
-                                         a.KVH, a.D, a.page, a.scale, a.window, stream);
+                rc = tm_attn_prefill_f32_cap(q, q_stride, attn, HD, a.k_pool, a.v_pool, tables, W, s->prefill_tiles, s->n_tiles, a.H,
+                                             a.KVH, a.D, a.page, a.scale, a.window, a.softcap, stream);
                 done_prefill = true;
             }
             if (rc) return rc;
@@ -361,25 +367,31 @@ struct Run {
             char* out_dec = (char*)attn + (size_t)tp * HD * es;
             if (nd && dtype == TM_BF16 && head_mfma && page_ok && a.H / a.KVH <= 16 && q_ok) {
                 const bool split = tm_decode_splits(nd, a.KVH, s->max_decode_context);
-                rc = tm_attn_decode_mfma(q_dec, q_stride, out_dec, HD, a.k_pool, a.v_pool, tables + (size_t)(S - nd) * W, W,
-                                         s->context_lens + (S - nd), split ? part_o : nullptr, split ? part_ml : nullptr,
-                                         tm_decode_chunks(s->max_decode_context), nd, a.H, a.KVH, a.D, a.page, a.scale, a.window,
-                                         stream);
+                rc = tm_attn_decode_mfma_cap(q_dec, q_stride, out_dec, HD, a.k_pool, a.v_pool, tables + (size_t)(S - nd) * W, W,
+                                             s->context_lens + (S - nd), split ? part_o : nullptr, split ? part_ml : nullptr,
+                                             tm_decode_chunks(s->max_decode_context), nd, a.H, a.KVH, a.D, a.page, a.scale, a.window,
+                                             a.softcap, stream);
                 done_decode = true;
             }
             if (rc) return rc;
             if (tp && !done_prefill && nd && !done_decode) {
-                rc = tm_attn_paged_generic(q, q_stride, attn, HD, a.k_pool, a.v_pool, tables, W, s->seq_of_token, s->positions, T,
-                                           a.H, a.KVH, a.D, a.page, a.scale, a.window, dtype, stream);
+                rc = tm_attn_paged_generic_ext(q, q_stride, attn, HD, a.k_pool, a.v_pool, tables, W, s->seq_of_token, s->positions, T,
+                                               a.H, a.KVH, a.D, a.D, a.page, a.scale, a.window, a.softcap, nullptr, 0, dtype, stream);
             } else {
                 if (tp && !done_prefill)
-                    rc = tm_attn_paged_generic(q, q_stride, attn, HD, a.k_pool, a.v_pool, tables, W, s->seq_of_token, s->positions,
-                                               tp, a.H, a.KVH, a.D, a.page, a.scale, a.window, dtype, stream);
+                    rc = tm_attn_paged_generic_ext(q, q_stride, attn, HD, a.k_pool, a.v_pool, tables, W, s->seq_of_token, s->positions,
+                                                   tp, a.H, a.KVH, a.D, a.D, a.page, a.scale, a.window, a.softcap, nullptr, 0, dtype, stream);
                 if (!rc && nd && !done_decode)
-                    rc = tm_attn_paged_generic(q_dec, q_stride, out_dec, HD, a.k_pool, a.v_pool, tables, W, s->seq_of_token + tp,
-                                               s->positions + tp, nd, a.H, a.KVH, a.D, a.page, a.scale, a.window, dtype, stream);
+                    rc = tm_attn_paged_generic_ext(q_dec, q_stride, out_dec, HD, a.k_pool, a.v_pool, tables, W, s->seq_of_token + tp,
+                                                   s->positions + tp, nd, a.H, a.KVH, a.D, a.D, a.page, a.scale, a.window, a.softcap, nullptr, 0,
+                                                   dtype, stream);
             }
             if (rc) return rc;
+            if (gate_in) {                  // a gate per (token, head) on the way to the output projection
+                rc = tm_head_gate(attn, dtype, gate_in, gate_ld, T, a.H, a.D, stream);
+                gate_in = nullptr;
+                if (rc) return rc;
+            }
         }
         Label l(this, op, TM_LABEL_O_PROJ);
         return project(a.o, attn, HD, T);
@@ -497,14 +509,15 @@ int tm_program_add_embedding(TmProgram* p, const TmEmbedOp* e) {
 
 int tm_program_add_attention(TmProgram* p, const TmAttentionOp* a) {
     if (!p || !a || a->H <= 0 || a->KVH <= 0 || a->H % a->KVH || a->D <= 0 || !a->k_pool || !a->v_pool || a->page <= 0 ||
-        !linear_fits(p, a->qkv) || !linear_fits(p, a->o) || a->qkv.K != p->hidden || a->qkv.N != (a->H + 2 * a->KVH) * a->D || a->o.K != a->H * a->D || a->o.N != p->hidden ||
+        !linear_fits(p, a->o) || a->o.K != a->H * a->D || a->o.N != p->hidden || !(a->softcap >= 0.f) ||
+        (!a->outside && (!linear_fits(p, a->qkv) || a->qkv.K != p->hidden || a->qkv.N != (a->H + 2 * a->KVH) * a->D)) ||
         a->window < 0 || a->rot < 0 || a->rot > a->D || (a->rot > 0 && (!a->cos_t || !a->sin_t)))
         return -1;
     Op op{};
     op.kind = OP_ATTENTION;
     op.att = *a;
     p->ops.push_back(op);
-    if (a->qkv.N > p->max_qkv) p->max_qkv = a->qkv.N;
+    if (!a->outside && a->qkv.N > p->max_qkv) p->max_qkv = a->qkv.N;
     if (a->H > p->max_heads) p->max_heads = a->H;
     if (a->H * a->D > p->max_heads_d) p->max_heads_d = a->H * a->D;
     return (int)p->ops.size() - 1;
@@ -587,6 +600,8 @@ int tm_program_run(const TmProgram* p, int first, int count, const TmStep* s, Tm
     r.from_norm_rows = tm_from_norm_rows(p->hidden);
     r.labels = (flags & TM_RUN_LABELS) != 0;
     r.resid = io->resid; r.delta = io->delta; r.x_in = io->x; r.qkv_in = io->qkv; r.accumulate = io->accumulate != 0;
+    r.qkv_in_stride = io->qkv_stride; r.gate_in = io->qkv ? io->gate : nullptr; r.gate_ld = io->ldg;
+    if (r.gate_in && r.gate_ld < p->ops[first].att.H) return TM_ERR_ARG;
     r.x = take((size_t)T * p->hidden * es);
     r.qkv = take((size_t)T * p->max_qkv * es);
     r.attn = take((size_t)T * p->max_heads_d * es);

@@ -31,7 +31,7 @@ class TmAttentionOp(Structure):
     _fields_ = [("norm", TmNorm), ("qkv", TmLinear), ("o", TmLinear), ("cos_t", c_void_p), ("sin_t", c_void_p),
                 ("k_pool", c_void_p), ("v_pool", c_void_p), ("H", c_int), ("KVH", c_int), ("D", c_int), ("scale", c_float),
                 ("window", c_int), ("rot", c_int), ("max_positions", c_int), ("page", c_int), ("group", c_int),
-                ("write", c_int)]
+                ("write", c_int), ("softcap", c_float), ("outside", c_int)]
 
 
 class TmFfnOp(Structure):
@@ -51,7 +51,8 @@ class TmStep(Structure):
 
 
 class TmStream(Structure):
-    _fields_ = [("resid", c_void_p), ("delta", c_void_p), ("x", c_void_p), ("qkv", c_void_p), ("accumulate", c_int)]
+    _fields_ = [("resid", c_void_p), ("delta", c_void_p), ("x", c_void_p), ("qkv", c_void_p), ("accumulate", c_int),
+                ("qkv_stride", c_int), ("gate", c_void_p), ("ldg", c_int)]
 
 
 TmHook = CFUNCTYPE(None, c_void_p, c_int, c_int, c_int)

@@ -38,6 +38,7 @@ class Flow:
     logits: torch.Tensor | None = None       # float32 [R, vocab], set by the head
     x: torch.Tensor | None = None            # into a single operation: its input, already normed
     qkv: torch.Tensor | None = None          # into a single attention: q|k|v already projected, encoded and stored
+    gate: torch.Tensor | None = None         # with qkv: float32 [T, >= H], a gate per (token, head) on that attention's result
     accumulate: bool = True                  # may an operation add its result into resid itself?
     delta_norm: object | None = None         # a norm that delta passes before it is added (a block that norms its results)
 
@@ -142,10 +143,13 @@ class StepProgram:
         return self._added(self._lib.tm_program_add_embedding(self._handle, ctypes.byref(op)), part)
 
     def attention(self, part, norm, qkv, o, rotation, cache, num_heads: int, num_kv_heads: int, head_dim: int,
-                  scale: float, window: int | None) -> int | None:
+                  scale: float, window: int | None, softcap: float = 0.0) -> int | None:
         """resid += o(attention(rotate(qkv(norm(resid))))) over the paged cache ``cache`` (a ``KVCacheView``).
-        ``rotation``: (cos, sin, rotary width, positions) of a rotary encoding, or () for none."""
-        n, q, out = self._norm(norm), self._linear(qkv), self._linear(o)
+        ``rotation``: (cos, sin, rotary width, positions) of a rotary encoding, or () for none. ``softcap`` > 0: a scaled
+        score s becomes softcap * tanh(s / softcap). ``qkv`` None: the operation has no projection of its own and is only
+        ever handed q (its keys and values encoded and stored by the caller); ``norm`` is then not looked at."""
+        outside = qkv is None
+        n, q, out = self._norm(None if outside else norm), (TmLinear() if outside else self._linear(qkv)), self._linear(o)
         if n is None or q is None or out is None or getattr(cache, "k", None) is None or getattr(cache, "v", None) is None:
             return None
         if rotation:
@@ -157,7 +161,8 @@ class StepProgram:
             rot = n_pos = 0
         self._keep.append((cache.k, cache.v))
         op = TmAttentionOp(n, q, out, cos, sin, cache.k.data_ptr(), cache.v.data_ptr(), num_heads, num_kv_heads, head_dim,
-                           float(scale), window or 0, rot, n_pos, cache.k.shape[1], cache.group, 1 if cache.write else 0)
+                           float(scale), window or 0, rot, n_pos, cache.k.shape[1], cache.group, 1 if cache.write else 0,
+                           float(softcap or 0.0), 1 if outside else 0)
         return self._added(self._lib.tm_program_add_attention(self._handle, ctypes.byref(op)), part)
 
     def feed_forward(self, part, norm, gate_up, down, intermediate: int) -> int | None:
@@ -256,6 +261,13 @@ class StepProgram:
             if t is not None and (t.dtype != self.dtype or tuple(t.shape) != (T, self.hidden)):
                 raise ops.KernelArgumentError(f"{name} must be {self.dtype} [{T}, {self.hidden}]")
         io.accumulate = 1 if flow.accumulate and flow.resid is not None else 0
+        if flow.qkv is not None:
+            io.qkv_stride = flow.qkv.shape[1]
+            if flow.gate is not None:
+                g = flow.gate
+                if not g.is_cuda or g.dtype != torch.float32 or g.dim() != 2 or g.shape[0] != T or g.stride(1) != 1:
+                    raise ops.KernelArgumentError("a head gate is a float32 view [T, >= heads] with unit inner stride")
+                io.gate, io.ldg = g.data_ptr(), (g.stride(0) if T > 1 else max(g.stride(0), g.shape[1]))
         flags = (abi.RUN_LABELS if profiling.on() else 0) | (abi.RUN_TUNE_AT_ONCE if at_once else 0)
         lib_ws = ops.library_workspace(self.device)
         self._now = (step, T)
@@ -272,7 +284,7 @@ class StepProgram:
             raise ops.KernelArgumentError("the step program refused the step (a size or position a kernel does not run)")
         if rc != 0:
             raise RuntimeError(f"the step program failed (code {rc})")
-        flow.x = flow.qkv = None
+        flow.x = flow.qkv = flow.gate = None
         if io.delta:
             off = io.delta - workspace.data_ptr()
             n = T * self.hidden * torch.empty((), dtype=self.dtype).element_size()
@@ -301,10 +313,10 @@ class StepProgram:
             raise RuntimeError("the model's last part set no logits")
         return flow.logits
 
-    def run_one(self, op: int, step: "StepContext | None", *, resid=None, delta=None, x=None, qkv=None,
+    def run_one(self, op: int, step: "StepContext | None", *, resid=None, delta=None, x=None, qkv=None, gate=None,
                 accumulate: bool = False, rows: int | None = None) -> torch.Tensor | None:
         """One operation by itself (a part called from outside a program). Returns what it left to be added to the
         residual stream, or None if it added that itself (``accumulate``)."""
-        flow = Flow(resid=resid, delta=delta, x=x, qkv=qkv, accumulate=accumulate)
+        flow = Flow(resid=resid, delta=delta, x=x, qkv=qkv, gate=gate, accumulate=accumulate)
         self.run_ops(op, 1, step, flow, rows=rows)
         return flow.delta

@@ -21,6 +21,7 @@ import torch
 
 from tokenmill_amd import profiling
 from tokenmill_amd.hip import ops
+from tokenmill_amd.hip.program import StepProgram
 from tokenmill_amd.parts.base import KVCacheSpec, KVCacheView, Mixer, StepContext, as_tensor
 from tokenmill_amd.parts.linear import Linear
 from tokenmill_amd.parts.position import RotaryEmbedding
@@ -70,6 +71,7 @@ class SoftmaxAttention(Mixer):
         self.extra_names = extra_names
         self.q_norm: torch.Tensor | None = None
         self.k_norm: torch.Tensor | None = None
+        self._own: dict = {}                    # per cache: the library's attention operation as a program of its own
 
     def _linears(self):
         return [p for p in (self.proj, self.gate, self.o) if p is not None]
@@ -150,13 +152,32 @@ class SoftmaxAttention(Mixer):
                                       rot.cos if rot is not None else None, rot.sin if rot is not None else None,
                                       bool(rot is not None and rot.interleaved), step.positions, group.slot_mapping,
                                       cache.k if self.own_kv else None, cache.v if self.own_kv else None, has_kv=self.own_kv)
+        if D == Dv:
+            # keys and values of one size: the kernel library's own attention operation, which is handed q and chooses the
+            # kernels of a step (prompt portions and single tokens on the matrix unit where it takes the sizes), then
+            # gates the heads and projects
+            entry = self._library_op(cache, x.dtype)
+            if entry is not None:
+                program, op = entry
+                return program.run_one(op, step, qkv=q, gate=gate)
         out = torch.empty((T, H * Dv), dtype=x.dtype, device=x.device)
         with profiling.label("attention", lambda: self.cost("attention", step, T)):
             self._attend(q, out, gate, step, cache, group)
         with profiling.label("o_proj", lambda: self.o.cost(T)):
             return self.o.forward(out)
 
+    def _library_op(self, cache: KVCacheView, dtype):
+        key = (id(cache.k), dtype)
+        if key not in self._own:
+            program = StepProgram(dtype, self.hidden, cache.k.device)
+            op = program.attention(self, None, None, self.o, (), cache, self.num_heads, self.num_kv_heads, self.head_dim, self.scale,
+                                   self.window, self.softcap)
+            self._own[key] = (program, op, cache) if op is not None else None
+        entry = self._own[key]
+        return entry[:2] if entry is not None else None
+
     def _attend(self, q, out, gate, step: StepContext, cache: KVCacheView, group) -> None:
+        """Keys and values of different sizes: a token and a head a wavefront."""
         H, G, D, Dv = self.num_heads, self.num_kv_heads, self.head_dim, self.v_head_dim
         ops.attn_paged_softmax(q, out, cache.k, cache.v, group.block_tables, step.seq_of_token, step.positions, H, G, D, Dv,
                                self.scale, self.window or 0, self.softcap, gate)
