@@ -96,30 +96,44 @@ def project_kv(h, positions, kind: str, m: dict, t: dict, pre: str, eps, dtype):
     return rnd(k, dtype), rnd(v, dtype).view(-1, G, Dv)
 
 
-def attention(h, positions, kind: str, m: dict, t: dict, pre: str, eps, dtype, keys, values, key_positions):
-    """h [T, W]: the mixer's input at ``positions``; keys [J, G, D] / values [J, G, Dv] at ``key_positions`` (this call's
-    tokens included). Softmax over the keys at or before a query; ``attention_2`` has biases, neighbouring rotation pairs
-    and capped scores; ``attention`` has a gate per head."""
-    H, G, D, Dv = int(m["heads"]), int(m["kv_heads"]), int(m["dim"]), int(m["vdim"])
-    T = h.shape[0]
-    biased = kind == "attention_2"
-    q = linear(h, t[pre + "q"], t[pre + "q.b"] if biased else None, dtype)
-    q = (unit(q, eps) * t[pre + "q.norm"].float()).view(T, H, D)
-    rot = m.get("rot")
-    if rot and int(rot.get("dims", 0)):
-        q = rotate(q, positions, rot, interleaved=biased)
-    q = rnd(q, dtype)
+def attend(q, keys, values, positions, key_positions, scale, softcap=None, gate=None):
+    """q [T, H, D] at ``positions`` over keys [J, G, D] / values [J, G, Dv] at ``key_positions``: softmax over the keys at or
+    before a query of scale * q.k, capped to softcap * tanh(. / softcap) if ``softcap``; head h times sigmoid(gate[t, h])."""
+    H, G = q.shape[1], keys.shape[1]
     kk = keys.repeat_interleave(H // G, dim=1)
     vv = values.repeat_interleave(H // G, dim=1)
-    score = torch.einsum("thd,jhd->htj", q, kk) * float(m["scale"])
-    cap = m.get("softcap")
-    if cap:
-        score = float(cap) * torch.tanh(score / float(cap))
+    score = torch.einsum("thd,jhd->htj", q, kk) * float(scale)
+    if softcap:
+        score = float(softcap) * torch.tanh(score / float(softcap))
     seen = key_positions[None, :] <= positions[:, None]
     score = score.masked_fill(~seen[None], float("-inf"))
     o = torch.einsum("htj,jhd->thd", torch.softmax(score, -1), vv)
-    if pre + "g" in t:
-        o = o * torch.sigmoid(linear(h, t[pre + "g"], None, dtype))[:, :, None]
+    if gate is not None:
+        o = o * torch.sigmoid(gate)[:, :, None]
+    return o
+
+
+def project_q(h, positions, kind: str, m: dict, t: dict, pre: str, eps, dtype):
+    """Queries [T, H, D]: normed over the whole projection, rotated, rounded."""
+    H, D = int(m["heads"]), int(m["dim"])
+    biased = kind == "attention_2"
+    q = linear(h, t[pre + "q"], t[pre + "q.b"] if biased else None, dtype)
+    q = (unit(q, eps) * t[pre + "q.norm"].float()).view(-1, H, D)
+    rot = m.get("rot")
+    if rot and int(rot.get("dims", 0)):
+        q = rotate(q, positions, rot, interleaved=biased)
+    return rnd(q, dtype)
+
+
+def attention(h, positions, kind: str, m: dict, t: dict, pre: str, eps, dtype, keys, values, key_positions):
+    """h [T, W]: the mixer's input at ``positions``; keys [J, G, D] / values [J, G, Dv] at ``key_positions`` (this call's
+    tokens included). ``attention_2`` has biases, neighbouring rotation pairs and capped scores; ``attention`` has a gate
+    per head."""
+    H, Dv = int(m["heads"]), int(m["vdim"])
+    T = h.shape[0]
+    q = project_q(h, positions, kind, m, t, pre, eps, dtype)
+    gate = linear(h, t[pre + "g"], None, dtype) if pre + "g" in t else None
+    o = attend(q, keys, values, positions, key_positions, m["scale"], m.get("softcap"), gate)
     return linear(rnd(o, dtype).reshape(T, H * Dv), t[pre + "o"], None, dtype)
 
 
@@ -142,7 +156,7 @@ def route(h, mlp: dict, t: dict, pre: str, dtype):
 def experts(h, mlp: dict, t: dict, pre: str, dtype):
     """Routed experts (the last ``identity`` router outputs stand for the input itself), plus the shared expert times a
     sigmoid of one number a token."""
-    E = int(mlp["router"]["experts"])
+    E = int(mlp["router"]["experts"])             # router outputs E .. E + identity - 1 stand for the input itself
     chosen, w = route(h, mlp, t, pre, dtype)
     hr = rnd(h, dtype)
     out = torch.zeros_like(h)

@@ -589,8 +589,9 @@ def attn_decode_mfma_supported(dtype, H: int, KVH: int, D: int, page: int) -> bo
 def attn_decode_mfma(q: torch.Tensor, out: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor,
                      block_tables: torch.Tensor, context_lens: torch.Tensor, H: int, KVH: int, D: int, scale: float,
                      window: int, max_context: int, workspace: tuple[torch.Tensor, torch.Tensor] | None = None,
-                     split: bool | None = None):
-    """Attention of one new token per request over its cache (the token's own key included).
+                     split: bool | None = None, softcap: float = 0.0):
+    """Attention of one new token per request over its cache (the token's own key included); ``softcap`` > 0: a scaled
+    score s becomes softcap * tanh(s / softcap).
     q: [S, >= H*D] rows (unit inner stride), out [S, H*D] view; block_tables int32 [S, W];
     context_lens int32 [S] (new token counted); max_context >= every context length. ``split``: None runs
     the kernel the library's rule names for this many requests (contexts split over blocks and merged, or one
@@ -623,10 +624,10 @@ def attn_decode_mfma(q: torch.Tensor, out: torch.Tensor, k_pool: torch.Tensor, v
         _need(part_o.numel() >= S * H * chunks * D and part_ml.numel() >= S * H * chunks * 2
               and part_o.dtype == torch.float32 and part_ml.dtype == torch.float32, "attn_decode: workspace too small")
     _need(out_stride % 4 == 0 and out.data_ptr() % 8 == 0, "attn_decode: out rows must be 8-byte aligned")
-    _check(library().tm_attn_decode_mfma(_p(q), c_int(q_stride), _p(out), c_int(out_stride), _p(k_pool), _p(v_pool),
-                                         _p(block_tables), c_int(W), _p(context_lens), _p(part_o), _p(part_ml),
-                                         c_int(chunks), c_int(S), c_int(H), c_int(KVH), c_int(D), c_int(page),
-                                         c_float(scale), c_int(window), _stream()), "attn_decode_mfma")
+    _check(library().tm_attn_decode_mfma_cap(_p(q), c_int(q_stride), _p(out), c_int(out_stride), _p(k_pool), _p(v_pool),
+                                             _p(block_tables), c_int(W), _p(context_lens), _p(part_o), _p(part_ml),
+                                             c_int(chunks), c_int(S), c_int(H), c_int(KVH), c_int(D), c_int(page),
+                                             c_float(scale), c_int(window), c_float(softcap), _stream()), "attn_decode_mfma")
     return out
 
 
@@ -640,8 +641,8 @@ def attn_prefill_mfma_supported(dtype, H: int, KVH: int, D: int, page: int) -> b
 
 def attn_prefill_mfma(q: torch.Tensor, out: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor,
                       block_tables: torch.Tensor, tiles: torch.Tensor, H: int, KVH: int, D: int, scale: float,
-                      window: int, shared: bool = False) -> torch.Tensor:
-    """Attention of prompt portions over the cache. q: [T, >= H*D] rows, out [T, H*D]; tiles int32
+                      window: int, shared: bool = False, softcap: float = 0.0) -> torch.Tensor:
+    """Attention of prompt portions over the cache (``softcap`` > 0: a scaled score s becomes softcap * tanh(s / softcap)). q: [T, >= H*D] rows, out [T, H*D]; tiles int32
     [n, 4] = (request index, first row, tokens (1..16), position of the first token) cover the rows
     to compute; every row of a tile belongs to one request at consecutive positions. ``shared``: the kernel
     that stages a tile's keys and values through LDS for all heads of a kv head, instead of the one whose
@@ -664,11 +665,11 @@ def attn_prefill_mfma(q: torch.Tensor, out: torch.Tensor, k_pool: torch.Tensor, 
         _need(bool(library().tm_attn_prefill_shared_takes(c_int(H), c_int(KVH), c_int(D))) and out_stride % 4 == 0
               and out.data_ptr() % 8 == 0, "attn_prefill: the shared-keys kernel takes up to 16 query heads a kv head "
               "and out rows aligned to 8 bytes")
-    entry = library().tm_attn_prefill_shared if shared else library().tm_attn_prefill_mfma
+    entry = library().tm_attn_prefill_shared_cap if shared else library().tm_attn_prefill_mfma_cap
     _check(entry(_p(q), c_int(q_stride), _p(out), c_int(out_stride), _p(k_pool), _p(v_pool),
                  _p(block_tables), c_int(block_tables.shape[1]), _p(tiles),
                  c_int(tiles.shape[0]), c_int(H), c_int(KVH), c_int(D), c_int(page),
-                 c_float(scale), c_int(window), _stream()), "attn_prefill_shared" if shared else "attn_prefill_mfma")
+                 c_float(scale), c_int(window), c_float(softcap), _stream()), "attn_prefill_shared" if shared else "attn_prefill_mfma")
     return out
 
 
@@ -679,7 +680,7 @@ def attn_prefill_f32_supported(dtype, H: int, KVH: int, D: int, page: int) -> bo
 
 def attn_prefill_f32(q: torch.Tensor, out: torch.Tensor, k_pool: torch.Tensor, v_pool: torch.Tensor,
                      block_tables: torch.Tensor, tiles: torch.Tensor, H: int, KVH: int, D: int, scale: float,
-                     window: int) -> torch.Tensor:
+                     window: int, softcap: float = 0.0) -> torch.Tensor:
     """Attention of prompt portions over the cache in true 32-bit (32-bit MFMA). Operands as for
     ``attn_prefill_mfma``, all float32."""
     _gpu(q, out, k_pool, v_pool, block_tables, tiles)
@@ -696,10 +697,10 @@ def attn_prefill_f32(q: torch.Tensor, out: torch.Tensor, k_pool: torch.Tensor, v
           "attn_prefill_f32: block_tables must be contiguous int32 [S, W]")
     _need(tiles.dtype == torch.int32 and tiles.dim() == 2 and tiles.shape[1] == 4 and tiles.is_contiguous(),
           "attn_prefill_f32: tiles must be contiguous int32 [n, 4]")
-    _check(library().tm_attn_prefill_f32(_p(q), c_int(q_stride), _p(out), c_int(out_stride), _p(k_pool), _p(v_pool),
-                                         _p(block_tables), c_int(block_tables.shape[1]), _p(tiles),
-                                         c_int(tiles.shape[0]), c_int(H), c_int(KVH), c_int(D), c_int(page),
-                                         c_float(scale), c_int(window), _stream()), "attn_prefill_f32")
+    _check(library().tm_attn_prefill_f32_cap(_p(q), c_int(q_stride), _p(out), c_int(out_stride), _p(k_pool), _p(v_pool),
+                                             _p(block_tables), c_int(block_tables.shape[1]), _p(tiles),
+                                             c_int(tiles.shape[0]), c_int(H), c_int(KVH), c_int(D), c_int(page),
+                                             c_float(scale), c_int(window), c_float(softcap), _stream()), "attn_prefill_f32")
     return out
 
 

@@ -62,13 +62,14 @@ def build_gaborax(cfg: GaboraxConfig, max_positions: int | None = None) -> Decod
     embedding = TokenEmbedding(cfg.vocab_size, hidden, name="embed")
     tables: dict = {}
     layers, run = [], []
+    names = ("norm1", "mix.", "norm1", "norm2", "mlp.", "norm2")    # the pass-throughs in front have no tensors: the names are the norms' behind
     for i, layer in enumerate(cfg.layers):
         mixer = _mixer(cfg, layer, n_pos, tables)
         if layer.mlp is None:
-            layers.append(SandwichBlock(PassThrough(hidden), mixer, behind(), scales=("ls1", "ls2")))
+            layers.append(SandwichBlock(PassThrough(hidden), mixer, behind(), names=names, scales=("ls1", "ls2")))
         else:
             layers.append(SandwichBlock(PassThrough(hidden), mixer, behind(), PassThrough(hidden), _feed_forward(cfg, layer.mlp), behind(),
-                                        names=("norm1", "mix.", "norm1", "norm2", "mlp.", "norm2"), scales=("ls1", "ls2")))
+                                        names=names, scales=("ls1", "ls2")))
         src = layer.mixer.get("kv_from")
         run.append(LayerCall(i, cache_of=int(src) if src is not None else None))
     head = OutputHead(hidden, cfg.vocab_size, tied_to=embedding, name="head")
