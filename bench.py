@@ -3,7 +3,7 @@ weights, synthetic token ids, on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--dtype bfloat16|float32] [--layers L]
                     [--config CONFIG.json|NAME]      another shape of the architecture (7b, 32b, a file)
-                    [--part all|decode|prefill|offline|mixed7b|preempt32b|modinex|lusolix]
+                    [--part all|decode|prefill|offline|mixed7b|preempt32b|modinex|lusolix|gaborax]
                     [--part decode --contexts 8192,32768 --batches 8,64]     decode steps over long contexts
 
 A "step" is one decode step of the engine (scheduling, metadata upload, the forward pass and greedy
@@ -19,6 +19,7 @@ of their operations has to move and do), not from formulas of one architecture.
                         (portions of prompts beside decoding requests, budget 2,048), up to 64 at a time
     --part preempt32b   the 32B shape, context 8,192: 64 prompts of 2,048 ids on 8,192 pages of 16, so
                         that growth during decoding evicts requests; reports evictions and tok/s
+    --part gaborax      the Gaborax design at two such sizes (gaborax-1k, gaborax-2k) beside the same two Qwen2 models
     --part lusolix      the Lusolix design at two such sizes (lusolix-1k, lusolix-2k) beside the same two Qwen2 models
     --part modinex      the Modinex design at two sizes that resemble a real model's layers (shipped shapes modinex-1k,
                         modinex-2k), each beside the Qwen2 model of equal width, depth, heads and feed-forward
@@ -101,7 +102,7 @@ def main() -> int:
                     help="captured shapes also try every algorithm the library holds, not only its heuristic's candidates")
     ap.add_argument("--skip-points", action="store_true", help="only the headline batch and the prefill")
     ap.add_argument("--skip-kernels", action="store_true", help="no per-operation kernel trace")
-    ap.add_argument("--part", default="all", choices=["all", "decode", "prefill", "offline", "mixed7b", "preempt32b", "modinex", "lusolix"],
+    ap.add_argument("--part", default="all", choices=["all", "decode", "prefill", "offline", "mixed7b", "preempt32b", "modinex", "lusolix", "gaborax"],
                     help="all: the headline line. decode / prefill: only that (for profiling one of them). offline: "
                          "--requests prompts of --offline-prompt tokens submitted at once. mixed7b / preempt32b: see above")
     ap.add_argument("--requests", type=int, default=None, help="requests of the offline, mixed7b and preempt32b parts")
@@ -148,7 +149,7 @@ def main() -> int:
     # the position tables reach the longest context any engine of this run allows (each engine has its own limit)
     most_positions = max([max_model_len] + sweep + ([] if args.skip_points or args.part != "all" else list(LONG_POINTS)))
     most_positions = min(most_positions, shape.get("max_position_embeddings", most_positions))
-    model = None if args.part in ("modinex", "lusolix") else load_random_model(shape, seed=0, dtype=dtype, device=device, max_positions=most_positions)
+    model = None if args.part in ("modinex", "lusolix", "gaborax") else load_random_model(shape, seed=0, dtype=dtype, device=device, max_positions=most_positions)
     gen = torch.Generator().manual_seed(0)
     vocab = model.head.vocab if model is not None else None
 
@@ -367,7 +368,7 @@ def main() -> int:
                 "config": {**sizes(), "requests": n, "prompt": prompt_len, "gen": gen_tokens, "max_num_seqs": n,
                            "token_budget": 2048, "max_model_len": max_model_len, "block_size": BLOCK_SIZE, "pages": pages}}
 
-    if args.part in ("modinex", "lusolix"):
+    if args.part in ("modinex", "lusolix", "gaborax"):
         # the new design beside the closest existing model at equal size: the functions above measure whatever
         # `model` is, so each shape is loaded in turn
         rows = {}
