@@ -12,12 +12,12 @@
 #include "attention_prefill_common.h"
 
 #define GM_BN 64
-#define GM_BK 32
-#define GM_LD (GM_BK + 8)
+#define GM_BK 32            // k of a step through LDS (BK of the kernel): 32, or 128 for tiles of few rows, whose steps are
+                            // latency and not arithmetic: four times the bytes asked for at once, a quarter of the steps
 
 enum { GM_STORE = 0, GM_STORE_F32 = 1, GM_SILU_MUL = 2, GM_RELU2 = 3 };
 
-template <int RT, int MODE>
+template <int RT, int MODE, int BK = GM_BK>
 __global__ __launch_bounds__(256) void grouped_mfma_kernel(const bf16_t* __restrict__ A, int lda, int a_off,
                                                            const int* __restrict__ row_src, int src_div,
                                                            const bf16_t* __restrict__ W, void* __restrict__ Cv, int ldc, int c_off,
@@ -27,6 +27,7 @@ __global__ __launch_bounds__(256) void grouped_mfma_kernel(const bf16_t* __restr
                                                            const int* __restrict__ positions) {
     constexpr int BM = RT * 16;
     constexpr bool GATED = MODE == GM_SILU_MUL;
+    constexpr int GM_LD = BK + 8, PPR = BK / 8;                 // 16-byte pieces a row of a step
     __shared__ __align__(16) bf16_t As[BM][GM_LD];
     __shared__ __align__(16) bf16_t Bs[GATED ? 2 : 1][GM_BN][GM_LD];
     __shared__ int src[BM];
@@ -50,48 +51,58 @@ __global__ __launch_bounds__(256) void grouped_mfma_kernel(const bf16_t* __restr
     for (int t = 0; t < RT; ++t) acc[t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int t = 0; t < (GATED ? RT : 1); ++t) acu[t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-    // a thread's pieces of a k-step: RT / 4 of A (one if RT = 2 and the thread is among the first 128), one of W (two with
-    // a gate); those of the step after the current one are asked for before the current one is multiplied
-    constexpr int NA = (BM * 4 + 255) / 256;
-    u32x4_t ha[NA], hb, hu;
-    const int bn = threadIdx.x / 4, bc = threadIdx.x % 4;
+    // a thread's pieces of a k-step: NA of A and NB of W (twice that with a gate); those of the step after the current one are
+    // asked for before the current one is multiplied
+    constexpr int NA = (BM * PPR + 255) / 256, NB = GM_BN * PPR / 256;
+    u32x4_t ha[NA], hb[NB], hu[GATED ? NB : 1];
     auto fetch = [&](int k0) {
 #pragma unroll
         for (int u = 0; u < NA; ++u) {
-            const int idx = threadIdx.x + 256 * u, i = idx / 4, c = idx % 4;
+            const int idx = threadIdx.x + 256 * u, i = idx / PPR, c = idx % PPR;
             ha[u] = u32x4_t{0, 0, 0, 0};
-            if (idx < BM * 4 && src[i] >= 0 && k0 + 8 * c < K)
+            if (idx < BM * PPR && src[i] >= 0 && k0 + 8 * c < K)
                 ha[u] = *(const u32x4_t*)(A + (size_t)src[i] * lda + (size_t)group * a_off + k0 + 8 * c);
         }
-        const bool in = n0 + bn < N && k0 + 8 * bc < K;
-        hb = u32x4_t{0, 0, 0, 0};
-        if (in) hb = *(const u32x4_t*)(Wg + (size_t)(n0 + bn) * K + k0 + 8 * bc);
-        if (GATED) {
-            hu = u32x4_t{0, 0, 0, 0};
-            if (in) hu = *(const u32x4_t*)(Wg + (size_t)(N + n0 + bn) * K + k0 + 8 * bc);
+#pragma unroll
+        for (int u = 0; u < NB; ++u) {
+            const int idx = threadIdx.x + 256 * u, bn = idx / PPR, bc = idx % PPR;
+            const bool in = n0 + bn < N && k0 + 8 * bc < K;
+            hb[u] = u32x4_t{0, 0, 0, 0};
+            if (in) hb[u] = *(const u32x4_t*)(Wg + (size_t)(n0 + bn) * K + k0 + 8 * bc);
+            if (GATED) {
+                hu[u] = u32x4_t{0, 0, 0, 0};
+                if (in) hu[u] = *(const u32x4_t*)(Wg + (size_t)(N + n0 + bn) * K + k0 + 8 * bc);
+            }
         }
     };
     fetch(0);
-    for (int k0 = 0; k0 < K; k0 += GM_BK) {
+    for (int k0 = 0; k0 < K; k0 += BK) {
 #pragma unroll
         for (int u = 0; u < NA; ++u) {
             const int idx = threadIdx.x + 256 * u;
-            if (idx < BM * 4) *(u32x4_t*)&As[idx / 4][8 * (idx % 4)] = ha[u];
+            if (idx < BM * PPR) *(u32x4_t*)&As[idx / PPR][8 * (idx % PPR)] = ha[u];
         }
-        *(u32x4_t*)&Bs[0][bn][8 * bc] = hb;
-        if (GATED) *(u32x4_t*)&Bs[GATED ? 1 : 0][bn][8 * bc] = hu;
-        __syncthreads();
-        if (k0 + GM_BK < K) fetch(k0 + GM_BK);
-        PFrag bf, bu;
-        bf.u = *(const u32x4_t*)&Bs[0][16 * wave + r][8 * g];
-        if (GATED) bu.u = *(const u32x4_t*)&Bs[GATED ? 1 : 0][16 * wave + r][8 * g];
 #pragma unroll
-        for (int t = 0; t < RT; ++t) {
-            PFrag af;
-            af.u = *(const u32x4_t*)&As[16 * t + r][8 * g];
-            // rows of A as the first operand: the result holds C[row 4 g + i][column r]
-            acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af.b, bf.b, acc[t], 0, 0, 0);
-            if (GATED) acu[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af.b, bu.b, acu[t], 0, 0, 0);
+        for (int u = 0; u < NB; ++u) {
+            const int idx = threadIdx.x + 256 * u;
+            *(u32x4_t*)&Bs[0][idx / PPR][8 * (idx % PPR)] = hb[u];
+            if (GATED) *(u32x4_t*)&Bs[GATED ? 1 : 0][idx / PPR][8 * (idx % PPR)] = hu[u];
+        }
+        __syncthreads();
+        if (k0 + BK < K) fetch(k0 + BK);
+#pragma unroll
+        for (int kk = 0; kk < BK; kk += 32) {                   // k ascends in 32s whatever BK is: the same sums, bit for bit
+            PFrag bf, bu;
+            bf.u = *(const u32x4_t*)&Bs[0][16 * wave + r][kk + 8 * g];
+            if (GATED) bu.u = *(const u32x4_t*)&Bs[GATED ? 1 : 0][16 * wave + r][kk + 8 * g];
+#pragma unroll
+            for (int t = 0; t < RT; ++t) {
+                PFrag af;
+                af.u = *(const u32x4_t*)&As[16 * t + r][kk + 8 * g];
+                // rows of A as the first operand: the result holds C[row 4 g + i][column r]
+                acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af.b, bf.b, acc[t], 0, 0, 0);
+                if (GATED) acu[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af.b, bu.b, acu[t], 0, 0, 0);
+            }
         }
         __syncthreads();
     }
@@ -180,10 +191,10 @@ extern "C" int tm_moe_gate_up_mfma(const void* x, int ldx, const int* slot_pair,
     if (max_tiles == 0) return TM_OK;
     dim3 grid(max_tiles, (F + GM_BN - 1) / GM_BN);
     if (grid.y > 65535) return TM_ERR_ARG;
-#define GM_GO(RT_)                                                                                                             \
-    grouped_mfma_kernel<RT_, GM_SILU_MUL><<<grid, 256, 0, stream>>>((const bf16_t*)x, ldx, 0, slot_pair, top, (const bf16_t*)W, act, F, \
+#define GM_GO(RT_, BK_)                                                                                                             \
+    grouped_mfma_kernel<RT_, GM_SILU_MUL, BK_><<<grid, 256, 0, stream>>>((const bf16_t*)x, ldx, 0, slot_pair, top, (const bf16_t*)W, act, F, \
                                                                     0, nullptr, 0, tiles, n_tiles, 0, K, F, 0, 0, nullptr, nullptr, nullptr)
-    if (tile_rows == 32) GM_GO(2); else if (tile_rows == 64) GM_GO(4); else GM_GO(8);
+    if (tile_rows == 32) GM_GO(2, 128); else if (tile_rows == 64) GM_GO(4, GM_BK); else GM_GO(8, GM_BK);
 #undef GM_GO
     TM_CHECK_LAUNCH();
     return TM_OK;
@@ -199,10 +210,10 @@ extern "C" int tm_moe_up_act_mfma(const void* x, int ldx, const int* slot_pair, 
     if (max_tiles == 0) return TM_OK;
     dim3 grid(max_tiles, (F + GM_BN - 1) / GM_BN);
     if (grid.y > 65535) return TM_ERR_ARG;
-#define GM_GO(RT_)                                                                                                             \
-    grouped_mfma_kernel<RT_, GM_RELU2><<<grid, 256, 0, stream>>>((const bf16_t*)x, ldx, 0, slot_pair, top, (const bf16_t*)W, act, F, \
+#define GM_GO(RT_, BK_)                                                                                                             \
+    grouped_mfma_kernel<RT_, GM_RELU2, BK_><<<grid, 256, 0, stream>>>((const bf16_t*)x, ldx, 0, slot_pair, top, (const bf16_t*)W, act, F, \
                                                                  0, nullptr, 0, tiles, n_tiles, 0, K, F, 0, 0, nullptr, nullptr, nullptr)
-    if (tile_rows == 32) GM_GO(2); else if (tile_rows == 64) GM_GO(4); else GM_GO(8);
+    if (tile_rows == 32) GM_GO(2, 128); else if (tile_rows == 64) GM_GO(4, GM_BK); else GM_GO(8, GM_BK);
 #undef GM_GO
     TM_CHECK_LAUNCH();
     return TM_OK;
@@ -216,10 +227,10 @@ extern "C" int tm_moe_down_mfma(const void* act, const void* W, float* part, con
     if (max_tiles == 0) return TM_OK;
     dim3 grid(max_tiles, (N + GM_BN - 1) / GM_BN);
     if (grid.y > 65535) return TM_ERR_ARG;
-#define GM_GO(RT_)                                                                                                              \
-    grouped_mfma_kernel<RT_, GM_STORE_F32><<<grid, 256, 0, stream>>>((const bf16_t*)act, F, 0, nullptr, 1, (const bf16_t*)W, part, N, 0, \
+#define GM_GO(RT_, BK_)                                                                                                              \
+    grouped_mfma_kernel<RT_, GM_STORE_F32, BK_><<<grid, 256, 0, stream>>>((const bf16_t*)act, F, 0, nullptr, 1, (const bf16_t*)W, part, N, 0, \
                                                                      nullptr, 0, tiles, n_tiles, 0, F, N, 0, 0, nullptr, nullptr, nullptr)
-    if (tile_rows == 32) GM_GO(2); else if (tile_rows == 64) GM_GO(4); else GM_GO(8);
+    if (tile_rows == 32) GM_GO(2, 128); else if (tile_rows == 64) GM_GO(4, GM_BK); else GM_GO(8, GM_BK);
 #undef GM_GO
     TM_CHECK_LAUNCH();
     return TM_OK;

@@ -240,9 +240,9 @@ extern "C" int tm_moe_combine(const float* part, const int* pair_slot, void* y, 
 
 // ------------------------------------------------------------------------------------------------ a router
 
-#define RT_MAX_PER_LANE (MOE_MAX_EXPERTS / TM_WAVE)
-
-// A wavefront a token; lane l holds experts l, l + 64, ... Everything is 32-bit.
+// A wavefront a token; lane l holds experts l, l + 64, ... (RT_MAX_PER_LANE of them: 1, 4 or 16 by the number of experts).
+// Everything is 32-bit.
+template <int RT_MAX_PER_LANE>
 __global__ __launch_bounds__(TM_WAVE) void moe_router_kernel(const float* __restrict__ z, int ldz, const float* __restrict__ correction,
                                                              int E, int top, int* __restrict__ chosen, float* __restrict__ weight) {
     const int t = blockIdx.x, lane = threadIdx.x;
@@ -301,7 +301,9 @@ extern "C" int tm_moe_router(const float* z, int ldz, const float* correction, i
                              hipStream_t stream) {
     if (!z || !chosen || !weight || T < 0 || E <= 0 || E > MOE_MAX_EXPERTS || top <= 0 || top > E || ldz < E) return TM_ERR_ARG;
     if (T == 0) return TM_OK;
-    moe_router_kernel<<<T, TM_WAVE, 0, stream>>>(z, ldz, correction, E, top, chosen, weight);
+    if (E <= TM_WAVE) moe_router_kernel<1><<<T, TM_WAVE, 0, stream>>>(z, ldz, correction, E, top, chosen, weight);
+    else if (E <= 4 * TM_WAVE) moe_router_kernel<4><<<T, TM_WAVE, 0, stream>>>(z, ldz, correction, E, top, chosen, weight);
+    else moe_router_kernel<MOE_MAX_EXPERTS / TM_WAVE><<<T, TM_WAVE, 0, stream>>>(z, ldz, correction, E, top, chosen, weight);
     TM_CHECK_LAUNCH();
     return TM_OK;
 }

@@ -64,7 +64,7 @@ class SoftmaxAttention(Mixer):
         if self.gate_stacked:
             sizes.append(num_heads)
             stacked.append(extra_names[2])
-        self.proj = Linear(hidden, sizes, stacked, bias=qkv_bias, suffixes=suffixes)
+        self.proj = Linear(hidden, sizes, stacked, bias=qkv_bias, suffixes=suffixes, wide_bias=True)     # its result is taken in 32-bit
         self.gate = Linear(hidden, num_heads, extra_names[2], bias=False, suffixes=suffixes) if head_gate and not self.gate_stacked else None
         self.has_gate = head_gate
         self.o = Linear(num_heads * v_head_dim, hidden, names[3], bias=False, suffixes=suffixes)

@@ -15,7 +15,8 @@ from tokenmill_amd.weights.loader import TensorSpec
 
 class Linear(Part):
     def __init__(self, in_features: int, out_features: list[int] | int, names: list[str] | str,
-                 bias: bool = False, library_first: bool = False, suffixes: tuple[str, str] = (".weight", ".bias")):
+                 bias: bool = False, library_first: bool = False, suffixes: tuple[str, str] = (".weight", ".bias"),
+                 wide_bias: bool = False):
         self.in_features = in_features
         self.out_splits = [out_features] if isinstance(out_features, int) else list(out_features)
         self.names = [names] if isinstance(names, str) else list(names)
@@ -24,6 +25,7 @@ class Linear(Part):
         self.has_bias = bias
         self.bias_init_zero = False
         self.library_first = library_first              # a wide matrix the library reads fastest at any row count
+        self.wide_bias = wide_bias                      # the bias is kept in 32-bit (a product whose 32-bit result is wanted)
         self.suffixes = suffixes                        # what a checkpoint appends to a name for the matrix and for the bias
         self.weight: torch.Tensor | None = None
         self.bias: torch.Tensor | None = None
@@ -46,8 +48,8 @@ class Linear(Part):
         if self.has_bias:
             bs = [tensors[f"{prefix}{name}{sb}"] for name in self.names]
             self.bias = bs[0] if len(bs) == 1 else torch.cat(bs, dim=0).contiguous()
-            if self.weight.dtype == torch.float32 and self.bias.dtype != torch.float32:
-                self.bias = self.bias.float()          # a 32-bit product adds a 32-bit bias
+            if (self.weight.dtype == torch.float32 or self.wide_bias) and self.bias.dtype != torch.float32:
+                self.bias = self.bias.float()          # a 32-bit product, or one with a 32-bit result, adds a 32-bit bias
         self._desc = None
 
     def pack(self, rows, parts: list[int] | None = None) -> None:
