@@ -308,23 +308,24 @@ extern "C" int tm_moe_router(const float* z, int ldz, const float* correction, i
     return TM_OK;
 }
 
+// A block is a token and 256 columns: few tokens still make many blocks, and a thread's loads (the pair's slot, then its row)
+// wait once, not once a column.
 template <typename T>
 __global__ __launch_bounds__(256) void moe_combine_weighted_kernel(const float* __restrict__ part, const int* __restrict__ pair_slot,
                                                                    const float* __restrict__ weight, const T* __restrict__ x, int ldx,
                                                                    const float* __restrict__ shared, const float* __restrict__ shared_gate,
                                                                    int ldg, T* __restrict__ y, int top, int N) {
-    const int t = blockIdx.x;
+    const int t = blockIdx.x, c = blockIdx.y * 256 + threadIdx.x;
+    if (c >= N) return;
     const float sg = (shared && shared_gate) ? 1.f / (1.f + expf(-shared_gate[(size_t)t * ldg])) : 1.f;
-    for (int c = threadIdx.x; c < N; c += 256) {
-        float s = 0.f;
-        for (int k = 0; k < top; ++k) {
-            const int slot = pair_slot[t * top + k];
-            const float v = slot >= 0 ? part[(size_t)slot * N + c] : Elem<T>::load(x + (size_t)t * ldx + c);
-            s += weight[(size_t)t * top + k] * v;
-        }
-        if (shared) s += sg * shared[(size_t)t * N + c];
-        Elem<T>::store(y + (size_t)t * N + c, s);
+    float s = 0.f;
+    for (int k = 0; k < top; ++k) {
+        const int slot = pair_slot[t * top + k];
+        const float v = slot >= 0 ? part[(size_t)slot * N + c] : Elem<T>::load(x + (size_t)t * ldx + c);
+        s += weight[(size_t)t * top + k] * v;
     }
+    if (shared) s += sg * shared[(size_t)t * N + c];
+    Elem<T>::store(y + (size_t)t * N + c, s);
 }
 
 // shared (float32 [T, N]) and shared_gate (float32, one number a token, rows ldg apart) may be null.
@@ -334,11 +335,13 @@ extern "C" int tm_moe_combine_weighted(const float* part, const int* pair_slot, 
     if (!part || !pair_slot || !weight || !x || !y || T < 0 || top <= 0 || N <= 0 || ldx < N || (shared_gate && ldg < 1)) return TM_ERR_ARG;
     if (dtype != TM_F32 && dtype != TM_BF16) return TM_ERR_ARG;
     if (T == 0) return TM_OK;
+    const dim3 grid(T, (N + 255) / 256);
+    if (grid.y > 65535) return TM_ERR_ARG;
     if (dtype == TM_F32)
-        moe_combine_weighted_kernel<float><<<T, 256, 0, stream>>>(part, pair_slot, weight, (const float*)x, ldx, shared, shared_gate, ldg,
+        moe_combine_weighted_kernel<float><<<grid, 256, 0, stream>>>(part, pair_slot, weight, (const float*)x, ldx, shared, shared_gate, ldg,
                                                                   (float*)y, top, N);
     else
-        moe_combine_weighted_kernel<bf16_t><<<T, 256, 0, stream>>>(part, pair_slot, weight, (const bf16_t*)x, ldx, shared, shared_gate, ldg,
+        moe_combine_weighted_kernel<bf16_t><<<grid, 256, 0, stream>>>(part, pair_slot, weight, (const bf16_t*)x, ldx, shared, shared_gate, ldg,
                                                                    (bf16_t*)y, top, N);
     TM_CHECK_LAUNCH();
     return TM_OK;
