@@ -17,7 +17,7 @@
 
 enum { GM_STORE = 0, GM_STORE_F32 = 1, GM_SILU_MUL = 2, GM_RELU2 = 3 };
 
-template <int RT, int MODE, int BK = GM_BK>
+template <int RT, int MODE, int BK = GM_BK, int BN = GM_BN>
 __global__ __launch_bounds__(256) void grouped_mfma_kernel(const bf16_t* __restrict__ A, int lda, int a_off,
                                                            const int* __restrict__ row_src, int src_div,
                                                            const bf16_t* __restrict__ W, void* __restrict__ Cv, int ldc, int c_off,
@@ -28,8 +28,9 @@ __global__ __launch_bounds__(256) void grouped_mfma_kernel(const bf16_t* __restr
     constexpr int BM = RT * 16;
     constexpr bool GATED = MODE == GM_SILU_MUL;
     constexpr int GM_LD = BK + 8, PPR = BK / 8;                 // 16-byte pieces a row of a step
+    constexpr int NCG = BN / GM_BN;                             // groups of 64 columns a block: a wavefront has 16 columns of each
     __shared__ __align__(16) bf16_t As[BM][GM_LD];
-    __shared__ __align__(16) bf16_t Bs[GATED ? 2 : 1][GM_BN][GM_LD];
+    __shared__ __align__(16) bf16_t Bs[GATED ? 2 : 1][BN][GM_LD];
     __shared__ int src[BM];
     int group, row0, rows;
     if (tiles) {
@@ -38,7 +39,7 @@ __global__ __launch_bounds__(256) void grouped_mfma_kernel(const bf16_t* __restr
     } else {
         group = blockIdx.z, row0 = blockIdx.x * BM, rows = min(BM, T - row0);
     }
-    const int n0 = blockIdx.y * GM_BN;
+    const int n0 = blockIdx.y * BN;
     const int wave = threadIdx.x / TM_WAVE, lane = threadIdx.x % TM_WAVE, r = lane % 16, g = lane / 16;
     const bf16_t* Wg = W + (size_t)group * (GATED ? 2 : 1) * N * K;
     if (threadIdx.x < BM) {
@@ -46,14 +47,17 @@ __global__ __launch_bounds__(256) void grouped_mfma_kernel(const bf16_t* __restr
         src[i] = i < rows ? (row_src ? row_src[row0 + i] / src_div : row0 + i) : -1;
     }
     __syncthreads();
-    f32x4_t acc[RT], acu[GATED ? RT : 1];
+    f32x4_t acc[NCG][RT], acu[NCG][GATED ? RT : 1];
 #pragma unroll
-    for (int t = 0; t < RT; ++t) acc[t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    for (int cg = 0; cg < NCG; ++cg) {
 #pragma unroll
-    for (int t = 0; t < (GATED ? RT : 1); ++t) acu[t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+        for (int t = 0; t < RT; ++t) acc[cg][t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int t = 0; t < (GATED ? RT : 1); ++t) acu[cg][t] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    }
     // a thread's pieces of a k-step: NA of A and NB of W (twice that with a gate); those of the step after the current one are
     // asked for before the current one is multiplied
-    constexpr int NA = (BM * PPR + 255) / 256, NB = GM_BN * PPR / 256;
+    constexpr int NA = (BM * PPR + 255) / 256, NB = BN * PPR / 256;
     u32x4_t ha[NA], hb[NB], hu[GATED ? NB : 1];
     auto fetch = [&](int k0) {
 #pragma unroll
@@ -92,16 +96,23 @@ __global__ __launch_bounds__(256) void grouped_mfma_kernel(const bf16_t* __restr
         if (k0 + BK < K) fetch(k0 + BK);
 #pragma unroll
         for (int kk = 0; kk < BK; kk += 32) {                   // k ascends in 32s whatever BK is: the same sums, bit for bit
-            PFrag bf, bu;
-            bf.u = *(const u32x4_t*)&Bs[0][16 * wave + r][kk + 8 * g];
-            if (GATED) bu.u = *(const u32x4_t*)&Bs[GATED ? 1 : 0][16 * wave + r][kk + 8 * g];
+            PFrag bf[NCG], bu[NCG];
+#pragma unroll
+            for (int cg = 0; cg < NCG; ++cg) {
+                bf[cg].u = *(const u32x4_t*)&Bs[0][GM_BN * cg + 16 * wave + r][kk + 8 * g];
+                if (GATED) bu[cg].u = *(const u32x4_t*)&Bs[GATED ? 1 : 0][GM_BN * cg + 16 * wave + r][kk + 8 * g];
+            }
 #pragma unroll
             for (int t = 0; t < RT; ++t) {
                 PFrag af;
                 af.u = *(const u32x4_t*)&As[16 * t + r][kk + 8 * g];
-                // rows of A as the first operand: the result holds C[row 4 g + i][column r]
-                acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af.b, bf.b, acc[t], 0, 0, 0);
-                if (GATED) acu[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af.b, bu.b, acu[t], 0, 0, 0);
+                // rows of A as the first operand: the result holds C[row 4 g + i][column r]; a piece of A read from LDS
+                // meets every column group of the wavefront
+#pragma unroll
+                for (int cg = 0; cg < NCG; ++cg) {
+                    acc[cg][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af.b, bf[cg].b, acc[cg][t], 0, 0, 0);
+                    if (GATED) acu[cg][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af.b, bu[cg].b, acu[cg][t], 0, 0, 0);
+                }
             }
         }
         __syncthreads();
@@ -125,29 +136,32 @@ __global__ __launch_bounds__(256) void grouped_mfma_kernel(const bf16_t* __restr
             ((bf16_t*)Cv)[(size_t)row * ldc + (size_t)group * c_off + N + c] = A[(size_t)row * lda + (size_t)group * a_off + K + c];
         }
     }
-    const int n = n0 + 16 * wave + r;
-    if (n >= N) return;
 #pragma unroll
-    for (int t = 0; t < RT; ++t)
+    for (int cg = 0; cg < NCG; ++cg) {
+        const int n = n0 + GM_BN * cg + 16 * wave + r;
+        if (n >= N) continue;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int row = 16 * t + 4 * g + i;
-            if (row >= rows) continue;
-            const size_t at = (size_t)(row0 + row) * ldc + (size_t)group * c_off + n;
-            float v = acc[t][i];
-            if (MODE == GM_SILU_MUL) {
-                const float u = acu[t][i];
-                ((bf16_t*)Cv)[at] = f32_to_bf16(v / (1.0f + __expf(-v)) * u);
-            } else if (MODE == GM_RELU2) {
-                v = fmaxf(v, 0.f);
-                ((bf16_t*)Cv)[at] = f32_to_bf16(v * v);
-            } else if (MODE == GM_STORE_F32) {
-                ((float*)Cv)[at] = v;
-            } else {
-                if (gate) v *= 1.0f / (1.0f + __expf(-gate[(size_t)(row0 + row) * ldg + group]));
-                ((bf16_t*)Cv)[at] = f32_to_bf16(v);
+        for (int t = 0; t < RT; ++t)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int row = 16 * t + 4 * g + i;
+                if (row >= rows) continue;
+                const size_t at = (size_t)(row0 + row) * ldc + (size_t)group * c_off + n;
+                float v = acc[cg][t][i];
+                if (MODE == GM_SILU_MUL) {
+                    const float u = acu[cg][t][i];
+                    ((bf16_t*)Cv)[at] = f32_to_bf16(v / (1.0f + __expf(-v)) * u);
+                } else if (MODE == GM_RELU2) {
+                    v = fmaxf(v, 0.f);
+                    ((bf16_t*)Cv)[at] = f32_to_bf16(v * v);
+                } else if (MODE == GM_STORE_F32) {
+                    ((float*)Cv)[at] = v;
+                } else {
+                    if (gate) v *= 1.0f / (1.0f + __expf(-gate[(size_t)(row0 + row) * ldg + group]));
+                    ((bf16_t*)Cv)[at] = f32_to_bf16(v);
+                }
             }
-        }
+    }
 }
 
 static bool gm_aligned(const void* p) { return ((uintptr_t)p % 16) == 0; }
@@ -191,10 +205,11 @@ extern "C" int tm_moe_gate_up_mfma(const void* x, int ldx, const int* slot_pair,
     if (max_tiles == 0) return TM_OK;
     dim3 grid(max_tiles, (F + GM_BN - 1) / GM_BN);
     if (grid.y > 65535) return TM_ERR_ARG;
-#define GM_GO(RT_, BK_)                                                                                                             \
-    grouped_mfma_kernel<RT_, GM_SILU_MUL, BK_><<<grid, 256, 0, stream>>>((const bf16_t*)x, ldx, 0, slot_pair, top, (const bf16_t*)W, act, F, \
+#define GM_GO(RT_, BK_, BN_)                                                                                                             \
+    grouped_mfma_kernel<RT_, GM_SILU_MUL, BK_, BN_><<<dim3(max_tiles, (F + BN_ - 1) / BN_), 256, 0, stream>>>((const bf16_t*)x, ldx, 0, slot_pair, top, (const bf16_t*)W, act, F, \
                                                                     0, nullptr, 0, tiles, n_tiles, 0, K, F, 0, 0, nullptr, nullptr, nullptr)
-    if (tile_rows == 32) GM_GO(2, 128); else if (tile_rows == 64) GM_GO(4, GM_BK); else GM_GO(8, GM_BK);
+    // (64 columns a block whatever the tile: with a gate a wavefront holds two results a column)
+    if (tile_rows == 32) GM_GO(2, 128, GM_BN); else if (tile_rows == 64) GM_GO(4, GM_BK, GM_BN); else GM_GO(8, GM_BK, GM_BN);
 #undef GM_GO
     TM_CHECK_LAUNCH();
     return TM_OK;
@@ -210,10 +225,13 @@ extern "C" int tm_moe_up_act_mfma(const void* x, int ldx, const int* slot_pair, 
     if (max_tiles == 0) return TM_OK;
     dim3 grid(max_tiles, (F + GM_BN - 1) / GM_BN);
     if (grid.y > 65535) return TM_ERR_ARG;
-#define GM_GO(RT_, BK_)                                                                                                             \
-    grouped_mfma_kernel<RT_, GM_RELU2, BK_><<<grid, 256, 0, stream>>>((const bf16_t*)x, ldx, 0, slot_pair, top, (const bf16_t*)W, act, F, \
+#define GM_GO(RT_, BK_, BN_)                                                                                                             \
+    grouped_mfma_kernel<RT_, GM_RELU2, BK_, BN_><<<dim3(max_tiles, (F + BN_ - 1) / BN_), 256, 0, stream>>>((const bf16_t*)x, ldx, 0, slot_pair, top, (const bf16_t*)W, act, F, \
                                                                  0, nullptr, 0, tiles, n_tiles, 0, K, F, 0, 0, nullptr, nullptr, nullptr)
-    if (tile_rows == 32) GM_GO(2, 128); else if (tile_rows == 64) GM_GO(4, GM_BK); else GM_GO(8, GM_BK);
+    // tiles of 128 rows take 128 columns a block (a piece of A read from LDS meets two column groups) where that still
+    // leaves two blocks a CU to choose from
+    if (tile_rows == 32) GM_GO(2, 128, GM_BN); else if (tile_rows == 64) GM_GO(4, GM_BK, GM_BN);
+    else if ((long long)max_tiles * ((F + 127) / 128) >= 512) GM_GO(8, GM_BK, 128); else GM_GO(8, GM_BK, GM_BN);
 #undef GM_GO
     TM_CHECK_LAUNCH();
     return TM_OK;
@@ -227,10 +245,13 @@ extern "C" int tm_moe_down_mfma(const void* act, const void* W, float* part, con
     if (max_tiles == 0) return TM_OK;
     dim3 grid(max_tiles, (N + GM_BN - 1) / GM_BN);
     if (grid.y > 65535) return TM_ERR_ARG;
-#define GM_GO(RT_, BK_)                                                                                                              \
-    grouped_mfma_kernel<RT_, GM_STORE_F32, BK_><<<grid, 256, 0, stream>>>((const bf16_t*)act, F, 0, nullptr, 1, (const bf16_t*)W, part, N, 0, \
+#define GM_GO(RT_, BK_, BN_)                                                                                                              \
+    grouped_mfma_kernel<RT_, GM_STORE_F32, BK_, BN_><<<dim3(max_tiles, (N + BN_ - 1) / BN_), 256, 0, stream>>>((const bf16_t*)act, F, 0, nullptr, 1, (const bf16_t*)W, part, N, 0, \
                                                                      nullptr, 0, tiles, n_tiles, 0, F, N, 0, 0, nullptr, nullptr, nullptr)
-    if (tile_rows == 32) GM_GO(2, 128); else if (tile_rows == 64) GM_GO(4, GM_BK); else GM_GO(8, GM_BK);
+    // tiles of 128 rows take 128 columns a block (a piece of A read from LDS meets two column groups) where that still
+    // leaves two blocks a CU to choose from
+    if (tile_rows == 32) GM_GO(2, 128, GM_BN); else if (tile_rows == 64) GM_GO(4, GM_BK, GM_BN);
+    else if ((long long)max_tiles * ((N + 127) / 128) >= 512) GM_GO(8, GM_BK, 128); else GM_GO(8, GM_BK, GM_BN);
 #undef GM_GO
     TM_CHECK_LAUNCH();
     return TM_OK;
