@@ -65,8 +65,11 @@ __device__ __forceinline__ void store4<bf16_t>(bf16_t* dst, const float v[4], in
     }
 }
 
-__device__ __forceinline__ float bias_at(const void* bias, int bias_f32, int n) {
-    return bias_f32 ? ((const float*)bias)[n] : bf16_to_f32(((const bf16_t*)bias)[n]);
+// flags of a launch: the bias is 32-bit; the result is relu(.)^2 (after the bias, before the one rounding)
+enum { SK_BIAS_F32 = 1, SK_RELU2 = 2 };
+
+__device__ __forceinline__ float bias_at(const void* bias, int flags, int n) {
+    return (flags & SK_BIAS_F32) ? ((const float*)bias)[n] : bf16_to_f32(((const bf16_t*)bias)[n]);
 }
 
 // NT: tiles of 16 tokens. WAVES: wavefronts per block. SPLIT: they share a strip and split K.
@@ -79,7 +82,7 @@ __device__ __forceinline__ float bias_at(const void* bias, int bias_f32, int n) 
 template <int NT, int WAVES, bool SPLIT, bool SILU, typename TC, int ROWS = 16, bool PACKED = false>
 __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16_t* __restrict__ A, int lda,
                                                                  const bf16_t* __restrict__ W,
-                                                                 const void* __restrict__ bias, int bias_f32,
+                                                                 const void* __restrict__ bias, int flags,
                                                                  TC* __restrict__ C, int ldc, int M, int N, int K,
                                                                  float* __restrict__ accum, int ldacc,
                                                                  int up_strip0 = 0) {
@@ -199,7 +202,11 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16_t* _
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             float x = acc[0][t][i];
-            if (bias && nf + i < N) x += bias_at(bias, bias_f32, nf + i);
+            if (bias && nf + i < N) x += bias_at(bias, flags, nf + i);
+            if (!SILU && (flags & SK_RELU2)) {
+                x = fmaxf(x, 0.f);
+                x *= x;
+            }
             if (SILU) {
                 const float gt = bf16_to_f32(f32_to_bf16(x));
                 const float up = bf16_to_f32(f32_to_bf16(acc[1][t][i]));
@@ -224,7 +231,7 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_skinny_kernel(const bf16_t* _
 }
 
 template <int NT, bool SILU, typename TC>
-static int launch_skinny(const void* A, int lda, const void* W, const void* bias, int bias_f32, void* C, int ldc,
+static int launch_skinny(const void* A, int lda, const void* W, const void* bias, int flags, void* C, int ldc,
                          int M, int N, int K, float* accum, int ldacc, hipStream_t stream) {
     const int strips = (N + 15) / 16;
     if (NT == 1 && !SILU && strips < 192) {    // few rows and few tokens: short strips, so that every CU gets a block
@@ -232,7 +239,7 @@ static int launch_skinny(const void* A, int lda, const void* W, const void* bias
         const int n_strips = r8 ? (N + 7) / 8 : (N + 3) / 4;
 #define TM_SHORT(WV, RW)                                                                                         \
     gemm_skinny_kernel<1, WV, true, false, TC, RW><<<n_strips, 64 * WV, 0, stream>>>(                            \
-        (const bf16_t*)A, lda, (const bf16_t*)W, bias, bias_f32, (TC*)C, ldc, M, N, K, accum, ldacc)
+        (const bf16_t*)A, lda, (const bf16_t*)W, bias, flags, (TC*)C, ldc, M, N, K, accum, ldacc)
         if (K < 2048) {
             if (r8) TM_SHORT(4, 8); else TM_SHORT(4, 4);
         } else {
@@ -244,31 +251,32 @@ static int launch_skinny(const void* A, int lda, const void* W, const void* bias
     }
     if (strips >= 2048) {                      // many rows: a strip per wavefront
         gemm_skinny_kernel<NT, 4, false, SILU, TC><<<(strips + 3) / 4, 256, 0, stream>>>(
-            (const bf16_t*)A, lda, (const bf16_t*)W, bias, bias_f32, (TC*)C, ldc, M, N, K, accum, ldacc);
+            (const bf16_t*)A, lda, (const bf16_t*)W, bias, flags, (TC*)C, ldc, M, N, K, accum, ldacc);
     } else if (strips >= 256 || K < 2048) {    // a block of 4 wavefronts per strip
         gemm_skinny_kernel<NT, 4, true, SILU, TC><<<strips, 256, 0, stream>>>(
-            (const bf16_t*)A, lda, (const bf16_t*)W, bias, bias_f32, (TC*)C, ldc, M, N, K, accum, ldacc);
+            (const bf16_t*)A, lda, (const bf16_t*)W, bias, flags, (TC*)C, ldc, M, N, K, accum, ldacc);
     } else {                                   // few rows, long K: 16 wavefronts per strip
         gemm_skinny_kernel<NT, 16, true, SILU, TC><<<strips, 1024, 0, stream>>>(
-            (const bf16_t*)A, lda, (const bf16_t*)W, bias, bias_f32, (TC*)C, ldc, M, N, K, accum, ldacc);
+            (const bf16_t*)A, lda, (const bf16_t*)W, bias, flags, (TC*)C, ldc, M, N, K, accum, ldacc);
     }
     TM_CHECK_LAUNCH();
     return TM_OK;
 }
 
 template <bool SILU, typename TC>
-static int launch_skinny_nt(const void* A, int lda, const void* W, const void* bias, int bias_f32, void* C, int ldc,
+static int launch_skinny_nt(const void* A, int lda, const void* W, const void* bias, int flags, void* C, int ldc,
                             int M, int N, int K, float* accum, int ldacc, hipStream_t stream) {
     switch ((M + 15) / 16) {
-        case 1: return launch_skinny<1, SILU, TC>(A, lda, W, bias, bias_f32, C, ldc, M, N, K, accum, ldacc, stream);
-        case 2: return launch_skinny<2, SILU, TC>(A, lda, W, bias, bias_f32, C, ldc, M, N, K, accum, ldacc, stream);
-        case 3: return launch_skinny<3, SILU, TC>(A, lda, W, bias, bias_f32, C, ldc, M, N, K, accum, ldacc, stream);
-        case 4: return launch_skinny<4, SILU, TC>(A, lda, W, bias, bias_f32, C, ldc, M, N, K, accum, ldacc, stream);
+        case 1: return launch_skinny<1, SILU, TC>(A, lda, W, bias, flags, C, ldc, M, N, K, accum, ldacc, stream);
+        case 2: return launch_skinny<2, SILU, TC>(A, lda, W, bias, flags, C, ldc, M, N, K, accum, ldacc, stream);
+        case 3: return launch_skinny<3, SILU, TC>(A, lda, W, bias, flags, C, ldc, M, N, K, accum, ldacc, stream);
+        case 4: return launch_skinny<4, SILU, TC>(A, lda, W, bias, flags, C, ldc, M, N, K, accum, ldacc, stream);
         default: return TM_ERR_ARG;
     }
 }
 
 // silu == 0: C[M, N] = A W^T + bias, W [N, K].   silu == 1: C[M, N] = silu(A Wg^T) * (A Wu^T), W = [Wg; Wu] [2N, K].
+// silu == 2: C[M, N] = relu(A W^T + bias)^2.
 // A, W bfloat16; C bfloat16 (out_dtype 1) or float32 (0); bias bfloat16 or float32 or null.
 // accum != null: nothing is stored to C; the bfloat16-rounded result is added to accum[M, N] (float32, row
 // stride ldacc) instead: the residual add of the layer, done by the product that feeds it.
@@ -277,17 +285,19 @@ extern "C" int tm_gemm_skinny(const void* A, int lda, const void* W, const void*
                               int ldc, int M, int N, int K, int out_dtype, int silu, float* accum, int ldacc,
                               hipStream_t stream) {
     if (M <= 0 || N <= 0) return TM_OK;
+    const int relu2 = silu == 2;            // silu == 2: no second matrix, the result is relu(A W^T + bias)^2
+    if (relu2) silu = 0;
     if (accum && (silu || ldacc < N)) return TM_ERR_ARG;
     if (!accum && !C) return TM_ERR_ARG;
     if (M > 64 || K <= 0 || (K % 8) || (lda % 8) || lda < K || ldc < N || ((uintptr_t)A % 16) || ((uintptr_t)W % 16))
         return TM_ERR_ARG;
     if (silu && bias) return TM_ERR_ARG;
-    const int bias_f32 = bias_dtype == TM_F32;
+    const int flags = (bias_dtype == TM_F32 ? SK_BIAS_F32 : 0) | (relu2 ? SK_RELU2 : 0);    // the kernel's flags
     if (out_dtype == TM_BF16)
-        return silu ? launch_skinny_nt<true, bf16_t>(A, lda, W, bias, bias_f32, C, ldc, M, N, K, accum, ldacc, stream)
-                    : launch_skinny_nt<false, bf16_t>(A, lda, W, bias, bias_f32, C, ldc, M, N, K, accum, ldacc, stream);
+        return silu ? launch_skinny_nt<true, bf16_t>(A, lda, W, bias, flags, C, ldc, M, N, K, accum, ldacc, stream)
+                    : launch_skinny_nt<false, bf16_t>(A, lda, W, bias, flags, C, ldc, M, N, K, accum, ldacc, stream);
     if (out_dtype == TM_F32 && !silu)
-        return launch_skinny_nt<false, float>(A, lda, W, bias, bias_f32, C, ldc, M, N, K, accum, ldacc, stream);
+        return launch_skinny_nt<false, float>(A, lda, W, bias, flags, C, ldc, M, N, K, accum, ldacc, stream);
     return TM_ERR_ARG;
 }
 
@@ -300,12 +310,12 @@ extern "C" int tm_skinny_strip_rows(int N, int K) {
 }
 
 template <bool SILU, typename TC, int ROWS>
-static int launch_skinny_packed(const void* A, int lda, const void* W, const void* bias, int bias_f32, void* C, int ldc,
+static int launch_skinny_packed(const void* A, int lda, const void* W, const void* bias, int flags, void* C, int ldc,
                                 int M, int N, int K, float* accum, int ldacc, int up_strip0, hipStream_t stream) {
     const int strips = (N + ROWS - 1) / ROWS;
 #define TM_PACKED(WV, SPL, BLOCKS)                                                                               \
     gemm_skinny_kernel<1, WV, SPL, SILU, TC, ROWS, true><<<BLOCKS, 64 * WV, 0, stream>>>(                        \
-        (const bf16_t*)A, lda, (const bf16_t*)W, bias, bias_f32, (TC*)C, ldc, M, N, K, accum, ldacc, up_strip0)
+        (const bf16_t*)A, lda, (const bf16_t*)W, bias, flags, (TC*)C, ldc, M, N, K, accum, ldacc, up_strip0)
     if (ROWS == 16 && strips >= 2048) TM_PACKED(4, false, (strips + 3) / 4);      // many rows: a strip per wavefront
     else if (K < 2048 || (ROWS == 16 && strips >= 256)) TM_PACKED(4, true, strips);
     else TM_PACKED(16, true, strips);
@@ -320,18 +330,20 @@ extern "C" int tm_gemm_skinny_packed(const void* A, int lda, const void* W, int 
                                      void* C, int ldc, int M, int N, int K, int out_dtype, int silu, float* accum,
                                      int ldacc, hipStream_t stream) {
     if (M <= 0 || N <= 0) return TM_OK;
+    const int relu2 = silu == 2;            // as in tm_gemm_skinny
+    if (relu2) silu = 0;
     if (accum && (silu || ldacc < N)) return TM_ERR_ARG;
     if (!accum && !C) return TM_ERR_ARG;
     if (M > 16 || K <= 0 || (K % 8) || (lda % 8) || lda < K || ldc < N || ((uintptr_t)A % 16) || ((uintptr_t)W % 16) ||
         (rows != 16 && rows != 8 && rows != 4) || (silu && (rows != 16 || bias)))
         return TM_ERR_ARG;
-    const int bias_f32 = bias_dtype == TM_F32;
+    const int flags = (bias_dtype == TM_F32 ? SK_BIAS_F32 : 0) | (relu2 ? SK_RELU2 : 0);    // the kernel's flags
     const int up_strip0 = (N + 15) / 16;
 #define TM_PACKED_ROWS(SILU_, TC_)                                                                               \
     switch (rows) {                                                                                              \
-        case 16: return launch_skinny_packed<SILU_, TC_, 16>(A, lda, W, bias, bias_f32, C, ldc, M, N, K, accum, ldacc, up_strip0, stream); \
-        case 8: if (!SILU_) return launch_skinny_packed<false, TC_, 8>(A, lda, W, bias, bias_f32, C, ldc, M, N, K, accum, ldacc, 0, stream); break; \
-        default: if (!SILU_) return launch_skinny_packed<false, TC_, 4>(A, lda, W, bias, bias_f32, C, ldc, M, N, K, accum, ldacc, 0, stream); break; \
+        case 16: return launch_skinny_packed<SILU_, TC_, 16>(A, lda, W, bias, flags, C, ldc, M, N, K, accum, ldacc, up_strip0, stream); \
+        case 8: if (!SILU_) return launch_skinny_packed<false, TC_, 8>(A, lda, W, bias, flags, C, ldc, M, N, K, accum, ldacc, 0, stream); break; \
+        default: if (!SILU_) return launch_skinny_packed<false, TC_, 4>(A, lda, W, bias, flags, C, ldc, M, N, K, accum, ldacc, 0, stream); break; \
     }
     if (out_dtype == TM_BF16) {
         if (silu) { TM_PACKED_ROWS(true, bf16_t) } else { TM_PACKED_ROWS(false, bf16_t) }

@@ -21,6 +21,7 @@ struct TmLinear {               // y = x W^T + b, W [N, K]
     int N, K;
     int dtype;                  // type of w
     int library_first;          // the owner asks for the library's product at any row count (an output head)
+    int act;                    // 0: none; 1: y = relu(x W^T + b)^2 (in the product's epilogue where its kernel has one)
 };
 
 struct TmNorm {                 // weight * round(x * rsqrt(mean(x^2) + eps)); w null: the operation has no norm of

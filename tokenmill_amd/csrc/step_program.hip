@@ -118,44 +118,52 @@ struct Products {
             if ((rc = linear(L, TM_F32, wide_in, L.K, M, wide_out, L.N, TM_F32))) return rc;
             return tm_convert(wide_out, TM_F32, out, TM_BF16, (long long)M * L.N, stream);
         }
+        // an activation behind the product (L.act: relu squared): in the epilogue of the kernels for few rows, a pass
+        // of its own behind the others
+        const int ep = L.act ? 2 : 0;
+        auto then_act = [&](int rc) {
+            if (rc || !L.act) return rc;
+            if (ldc != L.N) return (int)TM_ERR_ARG;
+            return tm_relu2(out, out, out_dtype, (long long)M * L.N, stream);
+        };
         if (L.packed_parts == 1 && packed_ok(L, x, ldx, M, dtype, skinny_rows) && !L.library_first)
             return tm_gemm_skinny_packed(x, ldx, L.packed, L.packed_rows, L.bias, L.bias_dtype, out, ldc, M, L.N, L.K,
-                                         out_dtype, 0, nullptr, 0, stream);
+                                         out_dtype, ep, nullptr, 0, stream);
         if (dtype != TM_BF16) {
             const bool plain32 = out_dtype == TM_F32 && (L.bias_dtype == TM_NONE || L.bias_dtype == TM_F32);
             if (plain32 && M <= TM_GEMV_F32_ROWS && L.K % 4 == 0 && ldx % 4 == 0 && aligned(x, 16) && aligned(L.w, 16))
-                return tm_gemv_f32((const float*)x, ldx, (const float*)L.w, (const float*)L.bias, (float*)out, ldc, M, L.N, L.K, stream);
+                return then_act(tm_gemv_f32((const float*)x, ldx, (const float*)L.w, (const float*)L.bias, (float*)out, ldc, M, L.N, L.K, stream));
             if (plain32 && tm_gemm_f32_mfma_fits(x, ldx, L.w, L.bias, out, ldc, M, L.N, L.K))
-                return tm_gemm_f32_mfma((const float*)x, ldx, (const float*)L.w, (const float*)L.bias, (float*)out, ldc, M, L.N, L.K, stream);
-            return tm_gemm_nt_tiled(x, ldx, L.w, L.bias, L.bias_dtype, out, ldc, M, L.N, L.K, dtype, out_dtype, stream);
+                return then_act(tm_gemm_f32_mfma((const float*)x, ldx, (const float*)L.w, (const float*)L.bias, (float*)out, ldc, M, L.N, L.K, stream));
+            return then_act(tm_gemm_nt_tiled(x, ldx, L.w, L.bias, L.bias_dtype, out, ldc, M, L.N, L.K, dtype, out_dtype, stream));
         }
         const bool skinny = skinny_ok(L, x, ldx, dtype);
         if (L.library_first) {
             const int rc = library(L, x, ldx, M, out, ldc, out_dtype);
-            if (rc != TM_ERR_UNSUPPORTED) return rc;
+            if (rc != TM_ERR_UNSUPPORTED) return then_act(rc);
         }
         if (skinny && M <= TM_SKINNY_ROWS)
-            return tm_gemm_skinny(x, ldx, L.w, L.bias, L.bias_dtype, out, ldc, M, L.N, L.K, out_dtype, 0, nullptr, 0, stream);
+            return tm_gemm_skinny(x, ldx, L.w, L.bias, L.bias_dtype, out, ldc, M, L.N, L.K, out_dtype, ep, nullptr, 0, stream);
         {
             const int rc = library(L, x, ldx, M, out, ldc, out_dtype);
-            if (rc != TM_ERR_UNSUPPORTED) return rc;
+            if (rc != TM_ERR_UNSUPPORTED) return then_act(rc);
         }
         if (skinny) {
             const int es = elem_size(dtype), eo = elem_size(out_dtype);
             for (int r0 = 0; r0 < M; r0 += TM_SKINNY_MAX_ROWS) {
                 const int m = M - r0 < TM_SKINNY_MAX_ROWS ? M - r0 : TM_SKINNY_MAX_ROWS;
                 const int rc = tm_gemm_skinny((const char*)x + (size_t)r0 * ldx * es, ldx, L.w, L.bias, L.bias_dtype,
-                                              (char*)out + (size_t)r0 * ldc * eo, ldc, m, L.N, L.K, out_dtype, 0, nullptr, 0, stream);
+                                              (char*)out + (size_t)r0 * ldc * eo, ldc, m, L.N, L.K, out_dtype, ep, nullptr, 0, stream);
                 if (rc) return rc;
             }
             return TM_OK;
         }
-        return tm_gemm_nt_tiled(x, ldx, L.w, L.bias, L.bias_dtype, out, ldc, M, L.N, L.K, dtype, out_dtype, stream);
+        return then_act(tm_gemm_nt_tiled(x, ldx, L.w, L.bias, L.bias_dtype, out, ldc, M, L.N, L.K, dtype, out_dtype, stream));
     }
 
     // Is there a kernel that adds round(x W^T + b) into a 32-bit accumulator in its epilogue?
     bool accumulates(const TmLinear& L, int dtype, const void* x, int ldx, int M) const {
-        if (L.dtype != dtype || M <= 0) return false;
+        if (L.dtype != dtype || M <= 0 || L.act) return false;
         return (L.packed_parts == 1 && packed_ok(L, x, ldx, M, dtype, skinny_rows)) ||
                (M <= TM_SKINNY_ROWS && skinny_ok(L, x, ldx, dtype));
     }

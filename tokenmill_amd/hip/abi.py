@@ -16,7 +16,7 @@ class TmTune(Structure):
 
 class TmLinear(Structure):
     _fields_ = [("w", c_void_p), ("packed", c_void_p), ("bias", c_void_p), ("packed_rows", c_int), ("packed_parts", c_int),
-                ("bias_dtype", c_int), ("N", c_int), ("K", c_int), ("dtype", c_int), ("library_first", c_int)]
+                ("bias_dtype", c_int), ("N", c_int), ("K", c_int), ("dtype", c_int), ("library_first", c_int), ("act", c_int)]
 
 
 class TmNorm(Structure):

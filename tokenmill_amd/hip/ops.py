@@ -428,7 +428,8 @@ def pack_weight(w: torch.Tensor, rows: int, parts: list[int] | None = None) -> P
     return PackedWeight(data, N, K, rows, tuple(parts))
 
 
-def linear_desc(w: torch.Tensor, packed: "PackedWeight | None", bias: torch.Tensor | None, library_first: bool = False):
+def linear_desc(w: torch.Tensor, packed: "PackedWeight | None", bias: torch.Tensor | None, library_first: bool = False,
+                relu2: bool = False):
     """A matrix as the library's product rule takes it (a ``TmLinear``; the caller keeps the tensors alive)."""
     from tokenmill_amd.hip.abi import TmLinear
     _gpu(w, bias)
@@ -441,7 +442,7 @@ def linear_desc(w: torch.Tensor, packed: "PackedWeight | None", bias: torch.Tens
     return TmLinear(w.data_ptr(), packed.data.data_ptr() if packed is not None else None,
                     bias.data_ptr() if bias is not None else None, packed.rows if packed is not None else 0,
                     len(packed.parts) if packed is not None else 0, code(bias.dtype) if bias is not None else -1,
-                    w.shape[0], w.shape[1], code(w.dtype), 1 if library_first else 0)
+                    w.shape[0], w.shape[1], code(w.dtype), 1 if library_first else 0, 1 if relu2 else 0)
 
 
 def _linear_input(desc, x: torch.Tensor) -> int:

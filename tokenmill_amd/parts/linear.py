@@ -16,7 +16,7 @@ from tokenmill_amd.weights.loader import TensorSpec
 class Linear(Part):
     def __init__(self, in_features: int, out_features: list[int] | int, names: list[str] | str,
                  bias: bool = False, library_first: bool = False, suffixes: tuple[str, str] = (".weight", ".bias"),
-                 wide_bias: bool = False):
+                 wide_bias: bool = False, activation: str | None = None):
         self.in_features = in_features
         self.out_splits = [out_features] if isinstance(out_features, int) else list(out_features)
         self.names = [names] if isinstance(names, str) else list(names)
@@ -26,6 +26,9 @@ class Linear(Part):
         self.bias_init_zero = False
         self.library_first = library_first              # a wide matrix the library reads fastest at any row count
         self.wide_bias = wide_bias                      # the bias is kept in 32-bit (a product whose 32-bit result is wanted)
+        if activation not in (None, "relu2"):
+            raise ValueError(f"activation '{activation}' is not one a product applies itself (relu2)")
+        self.activation = activation                    # y = relu(x W^T + b)^2: in the product's epilogue where its kernel has one
         self.suffixes = suffixes                        # what a checkpoint appends to a name for the matrix and for the bias
         self.weight: torch.Tensor | None = None
         self.bias: torch.Tensor | None = None
@@ -74,7 +77,7 @@ class Linear(Part):
         change); None while there is nothing on a GPU to describe."""
         if self._desc is None and self.weight is not None and self.weight.is_cuda and self.weight.is_contiguous() \
                 and self.weight.dtype in (torch.float32, torch.bfloat16):
-            self._desc = ops.linear_desc(self.weight, self.packed, self.bias, self.library_first)
+            self._desc = ops.linear_desc(self.weight, self.packed, self.bias, self.library_first, relu2=self.activation == "relu2")
         return self._desc
 
     def cost(self, rows: int, in_bytes: int | None = None, out_bytes: int | None = None) -> tuple[int, int]:

@@ -112,7 +112,7 @@ class RoutedExperts(FeedForward):
             rows.append(1)
             stacked.append(shared_gate_name)
         self.router = Linear(hidden, rows, stacked, bias=False, suffixes=("", ".b"))
-        self.shared_up = Linear(hidden, shared_ff, shared_prefix + names[0], bias=False, suffixes=("", ".b")) if shared_ff else None
+        self.shared_up = Linear(hidden, shared_ff, shared_prefix + names[0], bias=False, suffixes=("", ".b"), activation="relu2") if shared_ff else None
         self.shared_down = Linear(shared_ff, hidden, shared_prefix + names[1], bias=False, suffixes=("", ".b")) if shared_ff else None
         self.up: torch.Tensor | None = None             # [E, F, hidden]
         self.down: torch.Tensor | None = None           # [E, hidden, F]
@@ -174,8 +174,7 @@ class RoutedExperts(FeedForward):
         shared = None
         if self.shared_up is not None:
             with profiling.label("shared", lambda: self.cost("shared", step, T)):
-                a = self.shared_up.forward(x)
-                ops.relu2(a, a)
+                a = self.shared_up.forward(x)                   # with the activation (the product's own epilogue or pass)
                 shared = self.shared_down.forward(a, out_dtype=torch.float32)
         with profiling.label("experts", lambda: self.cost("experts", step, T)):
             mfma = x.dtype == torch.bfloat16 and self.hidden % 8 == 0 and self.intermediate % 8 == 0 and x.stride(0) % 8 == 0
