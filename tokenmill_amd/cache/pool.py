@@ -5,7 +5,7 @@ page_size, kv_heads, head_dim], the reference's layout (reference
 src/infer/kv/paged_cache.py:1-6,28-34), and values [cache layers, pages, kv_heads, value size,
 page_size] (the value size is the head size unless a group's spec says otherwise): inside a page the values lie key-contiguous for each (head, d), which is the operand
 layout of the MFMA attention kernels (no transposition through LDS). Per state-holding layer one
-tensor [slots, *shape].
+tensor [slots, *shape] for each state it keeps.
 """
 from __future__ import annotations
 
@@ -49,17 +49,29 @@ class CachePools:
         for g, calls in enumerate(members):
             for idx, j in enumerate(calls):
                 views[j] = KVCacheView(self.k[g][idx], self.v[g][idx] if self.v[g] is not None else None, g, True)
+        def make(spec: StateSpec) -> torch.Tensor:
+            # one row more than there are slots: where the padding rows of a replayed step put their state
+            return torch.zeros((num_state_slots + 1, *spec.shape), dtype=spec.dtype or dtype, device=device)
+
         for j, spec in enumerate(specs):
             beside = isinstance(spec, LayerCacheSpec)
             if beside:
                 spec = spec.state
             if isinstance(spec, StateSpec):
-                # one row more than there are slots: where the padding rows of a replayed step put their state
-                self.states[j] = torch.zeros((num_state_slots + 1, *spec.shape), dtype=spec.dtype or dtype, device=device)
-                if beside and views[j] is not None:
-                    views[j].state = self.states[j]
-                else:
-                    views[j] = StateView(self.states[j])
+                held = self.states[j] = make(spec)
+            elif isinstance(spec, tuple) and spec:
+                # a layer that keeps several states (a recurrence's matrix and a convolution's last rows): one tensor each,
+                # handed to the layer as a tuple; the first stands under the call's index, the others beside it
+                held = tuple(make(s) for s in spec)
+                self.states[j] = held[0]
+                for n, t in enumerate(held[1:], 1):
+                    self.states[(j, n)] = t
+            else:
+                continue
+            if beside and views[j] is not None:
+                views[j].state = held
+            else:
+                views[j] = StateView(held)
         for j, call in enumerate(model.run):
             if call.cache_of is not None:
                 src = views[call.cache_of]

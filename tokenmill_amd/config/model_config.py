@@ -462,6 +462,147 @@ class GaboraxConfig:
                     raise ConfigError(f"layers[{i}]: shared.ff must be positive")
 
 
+@dataclass(frozen=True)
+class LuzevikLayer:
+    type: str                       # "latent_attention" | "parallel"
+    mixer: dict                     # the mixer's sizes and constants, as config.json gives them
+    mlp: dict | None                # {"kind": "dense", "ff"} | {"kind": "moe", "ff", "experts", "top"} | None
+
+
+@dataclass
+class LuzevikConfig:
+    """The Luzevik decoder: token embedding times a constant; layers whose sublayers read the residual stream itself and whose
+    results pass an RMS norm (plain weight) on their way into it; a mixer that is either attention through a shared latent
+    (queries through a latent of their own, rotation of pairs half the rotated width apart, a sink per head in the softmax,
+    possibly on another layer's cached rows) or two mixers side by side, softmax attention over grouped heads (biases,
+    per-head norm of q and k, linearly scaled rotation) and a gated delta rule behind short convolutions; a feed-forward
+    that is dense with a tanh-GELU gate or a set of routed SwiGLU experts (router with a bias, softmax over the chosen
+    logits); the output head is the embedding table. Every size and constant that can differ between two models is read
+    from config.json; the model has no position limit of its own (``max_positions`` if the file gives one)."""
+
+    vocab_size: int
+    hidden_size: int
+    norm_eps: float
+    embedding_scale: float
+    layers: tuple[LuzevikLayer, ...]
+    max_position_embeddings: int | None = None
+    eos_token_ids: tuple[int, ...] = field(default_factory=tuple)
+
+    architecture = "Luzevik"
+    MIXERS = ("latent_attention", "parallel")
+
+    @property
+    def num_hidden_layers(self) -> int:
+        return len(self.layers)
+
+    @classmethod
+    def from_dict(cls, raw: dict, generation: dict | None = None) -> "LuzevikConfig":
+        norm = _require(raw, "norm")
+        layers = []
+        for i, entry in enumerate(_require(raw, "layers")):
+            kind = entry.get("type")
+            if kind not in cls.MIXERS:
+                raise ConfigError(f"layers[{i}]: type '{kind}' is not one of {list(cls.MIXERS)}")
+            mixer = entry.get("mixer")
+            if not isinstance(mixer, dict):
+                raise ConfigError(f"layers[{i}] has no 'mixer' sizes")
+            if kind == "latent_attention":
+                wanted = [(mixer, k, "latent attention") for k in ("heads", "dim", "rot_dim", "vdim", "q_rank", "kv_rank", "scale")]
+            else:
+                left, right = mixer.get("left"), mixer.get("right")
+                if not isinstance(left, dict) or not isinstance(right, dict):
+                    raise ConfigError(f"layers[{i}]: a parallel mixer has 'left' and 'right' sizes")
+                wanted = [(left, k, "left mixer") for k in ("heads", "kv_heads", "dim", "vdim", "scale")] + \
+                    [(right, k, "right mixer") for k in ("heads", "kv_heads", "dim", "vdim", "conv")]
+            for where, key, what in wanted:
+                if where.get(key) is None:
+                    raise ConfigError(f"layers[{i}]: the {what} has no '{key}'")
+            mlp = entry.get("mlp")
+            if mlp is not None:
+                how = mlp.get("kind")
+                if how == "dense":
+                    if mlp.get("ff") is None:
+                        raise ConfigError(f"layers[{i}]: the dense feed-forward has no 'ff' width")
+                    mlp = {"kind": "dense", "ff": int(mlp["ff"])}
+                elif how == "moe":
+                    expert, router = mlp.get("expert") or {}, mlp.get("router") or {}
+                    for where, key in ((expert, "ff"), (router, "experts"), (router, "top")):
+                        if where.get(key) is None:
+                            raise ConfigError(f"layers[{i}]: the experts have no '{key}'")
+                    mlp = {"kind": "moe", "ff": int(expert["ff"]), "experts": int(router["experts"]), "top": int(router["top"])}
+                else:
+                    raise ConfigError(f"layers[{i}]: feed-forward kind '{how}' is not 'dense' or 'moe'")
+            layers.append(LuzevikLayer(kind, dict(mixer), mlp))
+        most = raw.get("max_positions")
+        cfg = cls(vocab_size=int(_require(raw, "vocab")), hidden_size=int(_require(raw, "width")), norm_eps=float(_require(norm, "eps")),
+                  embedding_scale=float(_require(_require(raw, "embedding"), "scale")), layers=tuple(layers),
+                  max_position_embeddings=int(most) if most is not None else None,
+                  eos_token_ids=collect_eos_ids(([generation] if generation else []) + [raw]))
+        cfg.validate()
+        return cfg
+
+    @staticmethod
+    def _check_rot(i: int, where: str, rot: dict | None, most: int, scaled: bool) -> None:
+        if not rot:
+            return
+        dims = int(rot.get("dims", 0))
+        if dims < 0 or dims % 2 or dims > most:
+            raise ConfigError(f"layers[{i}]: {where} rot.dims {dims} must be even and at most {most}")
+        if dims and not float(rot.get("base", 0)) > 0:
+            raise ConfigError(f"layers[{i}]: {where} rot.base must be positive")
+        sc = rot.get("scaling")
+        if sc:
+            if not scaled:
+                raise ConfigError(f"layers[{i}]: {where} rotation has no scaling")
+            if sc.get("factor") is None or not float(sc["factor"]) > 0:
+                raise ConfigError(f"layers[{i}]: {where} rot.scaling.factor must be positive")
+
+    def validate(self) -> None:
+        for name in ("vocab_size", "hidden_size"):
+            if getattr(self, name) <= 0:
+                raise ConfigError(f"{name} must be positive, got {getattr(self, name)}")
+        if self.max_position_embeddings is not None and self.max_position_embeddings <= 0:
+            raise ConfigError("max_positions must be positive")
+        if not self.norm_eps > 0:
+            raise ConfigError("norm.eps must be positive")
+        if not self.layers:
+            raise ConfigError("a model needs at least one layer")
+        for i, layer in enumerate(self.layers):
+            m = layer.mixer
+            if layer.type == "latent_attention":
+                for key in ("heads", "dim", "vdim", "q_rank", "kv_rank"):
+                    if int(m[key]) <= 0:
+                        raise ConfigError(f"layers[{i}]: {key} must be positive")
+                if int(m["rot_dim"]) < 0:
+                    raise ConfigError(f"layers[{i}]: rot_dim must not be negative")
+                self._check_rot(i, "the", m.get("rot"), int(m["rot_dim"]), scaled=False)
+                src = m.get("kv_from")
+                if src is not None:
+                    src = int(src)
+                    if not 0 <= src < i or self.layers[src].type != "latent_attention" or self.layers[src].mixer.get("kv_from") is not None:
+                        raise ConfigError(f"layers[{i}]: kv_from must name an earlier latent-attention layer that has a latent of its own")
+                    other = self.layers[src].mixer
+                    if any(int(other[k]) != int(m[k]) for k in ("kv_rank", "rot_dim")) or (other.get("rot") or {}) != (m.get("rot") or {}):
+                        raise ConfigError(f"layers[{i}]: layer {src}'s kv_rank, rot_dim and rotation must equal this layer's")
+            else:
+                for side in ("left", "right"):
+                    part = m[side]
+                    for key in ("heads", "kv_heads", "dim", "vdim"):
+                        if int(part[key]) <= 0:
+                            raise ConfigError(f"layers[{i}]: {side}.{key} must be positive")
+                    if int(part["heads"]) % int(part["kv_heads"]):
+                        raise ConfigError(f"layers[{i}]: {side}: {part['heads']} heads do not divide into {part['kv_heads']} kv_heads")
+                self._check_rot(i, "left", m["left"].get("rot"), int(m["left"]["dim"]), scaled=True)
+                if int(m["right"]["conv"]) < 1:
+                    raise ConfigError(f"layers[{i}]: right.conv must be at least 1")
+            mlp = layer.mlp
+            if mlp is not None:
+                if mlp["ff"] <= 0:
+                    raise ConfigError(f"layers[{i}]: the feed-forward's ff must be positive")
+                if mlp["kind"] == "moe" and not 0 < mlp["top"] <= mlp["experts"]:
+                    raise ConfigError(f"layers[{i}]: {mlp['top']} of {mlp['experts']} experts")
+
+
 def read_json(path: Path) -> dict:
     try:
         return json.loads(path.read_text())

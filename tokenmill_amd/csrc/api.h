@@ -67,7 +67,7 @@ int tm_attn_decode_mfma_cap(const void* q, int q_stride, void* out, int out_stri
 int tm_whole_norm_rope_store(const float* proj, int ld, void* q_out, int dtype, int T, int H, int G, int D, int Dv, int rot,
                              int interleaved, const float* q_w, const float* k_w, float eps, const float* cos_t, const float* sin_t,
                              const int* positions, const int* slots, void* k_pool, void* v_pool, int page, int has_kv,
-                             hipStream_t stream);
+                             int per_head, hipStream_t stream);
 int tm_head_gate(void* x, int dtype, const float* gate, int ldg, int T, int H, int Dv, hipStream_t stream);
 
 int tm_gemm_skinny(const void* A, int lda, const void* W, const void* bias, int bias_dtype, void* C, int ldc, int M,
@@ -214,17 +214,31 @@ int tm_short_conv_state(const void* h, void* state, const int* cu_q_lens, const 
 // out = a N(z) + b N(z^2) + c N(z^3) + e with coef = (a, b, c, e) on the device, N(v) = v / sqrt(mean(v^2) + eps) per row.
 int tm_poly_norm(const float* z, const float* coef, void* out, int dtype, int T, int F, float eps, hipStream_t stream);
 
+// The gated delta rule and two sublayers side by side (delta_rule.hip): see the head of that file.
+int tm_delta_prepare(const void* proj, int ld, const void* conv_w, const void* conv_state, const float* ba, int ldba,
+                     const float* a_log, const float* dt_bias, const int* cu_q_lens, const int* state_slots, const int* seq_of_token,
+                     float* out, int ldo, int T, int H, int G, int D, int Dv, int taps, float unit_eps, int dtype, hipStream_t stream);
+int tm_delta_conv_state(const void* proj, int ld, void* state, const int* cu_q_lens, const int* state_slots, int S, int C, int taps,
+                        int dtype, hipStream_t stream);
+int tm_delta_scan(const float* rows, int ld, float* o, float* state, const int* cu_q_lens, const int* state_slots, int S, int H, int G,
+                  int D, int Dv, hipStream_t stream);
+int tm_pair_norm_mean(const void* a, const void* b, const float* wa, const float* wb, void* out, int T, int W, float eps, int dtype,
+                      hipStream_t stream);
+int tm_gelu_mul(const void* gu, void* out, int dtype, int T, int I, hipStream_t stream);
+int tm_embed_gather_scaled(const void* table, int dtype, const int* ids, float* out, int T, int hidden, int vocab, float scale,
+                           hipStream_t stream);
+
 // Attention over a shared latent (latent.hip): see the head of that file.
 int tm_latent_prepare(const float* low, int ld, int Lq, int Lk, int Dr, int rot, const float* wq, const float* wk, float eps,
                       const float* cos_t, const float* sin_t, const int* positions, const int* slots, void* cq, void* pool,
-                      int dtype, int T, hipStream_t stream);
+                      int dtype, int T, int half_pairs, hipStream_t stream);
 int tm_heads_matmul(const void* A, int lda, int a_head, const void* B, void* C, int ldc, int c_head, const float* gate, int ldg,
                     int T, int H, int K, int N, int dtype, hipStream_t stream);
 int tm_rotate_heads(const void* src, int ld_src, int src_head, void* dst, int ld_dst, int dst_head, int T, int H, int Dr, int rot,
-                    const float* cos_t, const float* sin_t, const int* positions, int dtype, hipStream_t stream);
+                    const float* cos_t, const float* sin_t, const int* positions, int dtype, int half_pairs, hipStream_t stream);
 int tm_attn_latent(const void* qa, int q_stride, void* out, int out_stride, const void* pool, const int* block_tables,
                    int table_width, const int* seq_of_token, const int* positions, int T, int H, int Lk, int Dk, int page,
-                   float scale, int window, int dtype, hipStream_t stream);
+                   float scale, int window, const float* sink, int dtype, hipStream_t stream);
 // The same attention on the matrix unit (latent_mfma.hip), bfloat16: the prompt tiles of a step (tiles as for
 // tm_attn_prefill_mfma) or its single tokens (rows first_single .. first_single + n_single - 1), one of the two per call.
 int tm_attn_latent_mfma_takes(int Lk, int Dk, int q_stride, int out_stride);
@@ -236,7 +250,7 @@ int tm_attn_latent_chunks(int most_rows, int chunk_runs);
 int tm_attn_latent_mfma(const void* qa, int q_stride, void* out, int out_stride, const void* pool, const int* block_tables,
                         int table_width, const int* tiles, int n_tiles, const int* seq_of_token, const int* positions,
                         int first_single, int n_single, float* part_o, float* part_ml, int n_chunks, int chunk_runs, int H, int Lk,
-                        int Dk, int page, float scale, int window, hipStream_t stream);
+                        int Dk, int page, float scale, int window, const float* sink, hipStream_t stream);
 
 // Experts chosen by a table row of the token id (moe.hip): see the head of that file.
 int tm_moe_route(const int* ids, const int* table, int T, int top, int E, int tile_rows, int* slot_pair, int* pair_slot,
@@ -250,7 +264,7 @@ int tm_moe_combine(const float* part, const int* pair_slot, void* y, int T, int 
 
 // Experts chosen by a router, experts without a gate, experts that stand for the input itself, a shared expert (moe.hip).
 int tm_moe_router(const float* z, int ldz, const float* correction, int T, int E, int top, int* chosen, float* weight,
-                  hipStream_t stream);
+                  int over_chosen, hipStream_t stream);
 int tm_moe_route_chosen(const int* ids, const int* table, int T, int top, int E, int real, int tile_rows, int* slot_pair,
                         int* pair_slot, int* tiles, int* n_tiles, hipStream_t stream);
 int tm_moe_up_act(const void* x, int ldx, const int* slot_pair, int top, const void* W, void* act, const int* tiles,
@@ -265,7 +279,7 @@ int tm_moe_up_act_mfma(const void* x, int ldx, const int* slot_pair, int top, co
 int tm_heads_matmul_mfma_takes(const void* A, int lda, int a_off, const void* W, int K);
 int tm_heads_matmul_mfma(const void* A, int lda, int a_off, const void* W, void* C, int ldc, int c_off, const float* gate, int ldg,
                          int T, int H, int K, int N, int tail, int rot, const float* cos_t, const float* sin_t, const int* positions,
-                         hipStream_t stream);
+                         int half_pairs, hipStream_t stream);
 int tm_moe_mfma_takes(const void* x, int ldx, const void* Wgu, const void* Wd, const void* act, int K, int F);
 int tm_moe_gate_up_mfma(const void* x, int ldx, const int* slot_pair, int top, const void* W, void* act, const int* tiles,
                         const int* n_tiles, int max_tiles, int tile_rows, int K, int F, hipStream_t stream);

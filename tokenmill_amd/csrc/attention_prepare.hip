@@ -4,6 +4,7 @@
 //   proj row (32-bit) = [H heads of q, D wide | G heads of k, D wide | G heads of v, Dv wide | ...]   (k and v absent for a
 //                        layer that reads another layer's cache)
 //   qn = w_q * q / sqrt(mean(q^2 over all H * D) + eps), kn likewise over G * D with w_k      (weights null: no norm)
+//   with `per_head` every head of q and of k is normed by itself over its D channels, and w_q, w_k are [D], shared by the heads
 //   the first `rot` channels of every head of qn and kn turn by the token's position: pairs (j, j + rot/2), or neighbours
 //   (2j, 2j + 1) if `interleaved`; cos/sin [positions, rot/2] hold whatever frequencies and magnitude the model wants
 //   q goes to q_out [T, H * D] in the storage type; kn and v to the token's cache slot
@@ -15,26 +16,38 @@
 #include "api.h"
 
 #define AP_THREADS 256
+#define AP_MAX_HEADS 1024         // heads of q and k together that a token's per-head norms take
 
 template <typename T>
 __global__ __launch_bounds__(AP_THREADS) void whole_norm_rope_store_kernel(
     const float* __restrict__ proj, int ld, T* __restrict__ q_out, int H, int G, int D, int Dv, int rot, int interleaved,
     const float* __restrict__ q_w, const float* __restrict__ k_w, float eps, const float* __restrict__ cos_t,
     const float* __restrict__ sin_t, const int* __restrict__ positions, const int* __restrict__ slots, T* __restrict__ k_pool,
-    T* __restrict__ v_pool, int page, int has_kv) {
+    T* __restrict__ v_pool, int page, int has_kv, int per_head) {
     __shared__ float red[AP_THREADS / TM_WAVE];
+    __shared__ float inv_head[AP_MAX_HEADS];
     const int t = blockIdx.x;
     const float* row = proj + (size_t)t * ld;
     const int Q = H * D, K = has_kv ? G * D : 0;
     const int slot = (has_kv && slots) ? slots[t] : -1;
     const bool store = has_kv && k_pool && slot >= 0;
     float rq = 1.f, rk = 1.f;
-    if (q_w) {
+    const int heads = H + (has_kv ? G : 0);
+    if (per_head && q_w) {                      // a wavefront a head; a head's sum has one order per D
+        const int wave = threadIdx.x / TM_WAVE, lane = threadIdx.x % TM_WAVE;
+        for (int hh = wave; hh < heads; hh += AP_THREADS / TM_WAVE) {
+            float ss = 0.f;
+            for (int d = lane; d < D; d += TM_WAVE) ss += row[hh * D + d] * row[hh * D + d];
+            ss = wave_sum(ss);
+            if (lane == 0) inv_head[hh] = 1.0f / sqrtf(ss / (float)D + eps);
+        }
+        __syncthreads();
+    } else if (q_w) {
         float ss = 0.f;
         for (int c = threadIdx.x; c < Q; c += AP_THREADS) ss += row[c] * row[c];
         rq = 1.0f / sqrtf(block_sum<AP_THREADS>(ss, red) / (float)Q + eps);
     }
-    if (k_w && K) {
+    if (!per_head && k_w && K) {
         float ss = 0.f;
         for (int c = threadIdx.x; c < K; c += AP_THREADS) ss += row[Q + c] * row[Q + c];
         rk = 1.0f / sqrtf(block_sum<AP_THREADS>(ss, red) / (float)K + eps);
@@ -45,19 +58,19 @@ __global__ __launch_bounds__(AP_THREADS) void whole_norm_rope_store_kernel(
     T* qo = q_out + (size_t)t * Q;
     T* ko = store ? k_pool + (size_t)slot * G * D : nullptr;
     // the rotated pairs of every head of q and k
-    const int heads = H + (has_kv ? G : 0);
     for (int idx = threadIdx.x; idx < heads * half; idx += AP_THREADS) {
         const int hh = idx / half, j = idx % half;
         const int a = interleaved ? 2 * j : j, b = interleaved ? 2 * j + 1 : j + half;
         const int base = hh * D;                // q heads, then k heads, lie one behind the other in the row
         const bool is_q = hh < H;
         const float* w = is_q ? q_w : k_w;
-        const float r = is_q ? rq : rk;
+        const float r = per_head ? inv_head[hh] : is_q ? rq : rk;
         const int wb = is_q ? base : base - Q;
+        const int wi = per_head ? 0 : wb;       // where the head's weights start
         float x1 = row[base + a], x2 = row[base + b];
         if (w) {
-            x1 = w[wb + a] * (x1 * r);
-            x2 = w[wb + b] * (x2 * r);
+            x1 = w[wi + a] * (x1 * r);
+            x2 = w[wi + b] * (x2 * r);
         }
         float y1, y2;
         rotate_pair(x1, x2, cs[j], sn[j], y1, y2);
@@ -78,7 +91,7 @@ __global__ __launch_bounds__(AP_THREADS) void whole_norm_rope_store_kernel(
         const float* w = is_q ? q_w : k_w;
         const int wb = is_q ? base : base - Q;
         float x = row[base + d];
-        if (w) x = w[wb + d] * (x * (is_q ? rq : rk));
+        if (w) x = w[(per_head ? 0 : wb) + d] * (x * (per_head ? inv_head[hh] : is_q ? rq : rk));
         if (is_q) Elem<T>::store(qo + base + d, x);
         else if (ko) Elem<T>::store(ko + wb + d, x);
     }
@@ -93,8 +106,9 @@ __global__ __launch_bounds__(AP_THREADS) void whole_norm_rope_store_kernel(
 extern "C" int tm_whole_norm_rope_store(const float* proj, int ld, void* q_out, int dtype, int T, int H, int G, int D, int Dv,
                                         int rot, int interleaved, const float* q_w, const float* k_w, float eps,
                                         const float* cos_t, const float* sin_t, const int* positions, const int* slots,
-                                        void* k_pool, void* v_pool, int page, int has_kv, hipStream_t stream) {
+                                        void* k_pool, void* v_pool, int page, int has_kv, int per_head, hipStream_t stream) {
     if (T <= 0) return TM_OK;
+    if (per_head && H + G > AP_MAX_HEADS) return TM_ERR_ARG;
     if (!proj || !q_out || H <= 0 || G <= 0 || D <= 0 || Dv <= 0 || rot < 0 || rot > D || (rot & 1)) return TM_ERR_ARG;
     if (ld < H * D + (has_kv ? G * (D + Dv) : 0)) return TM_ERR_ARG;
     if ((q_w || k_w) && !(eps > 0.f)) return TM_ERR_ARG;
@@ -104,11 +118,11 @@ extern "C" int tm_whole_norm_rope_store(const float* proj, int ld, void* q_out, 
     if (dtype == TM_F32)
         whole_norm_rope_store_kernel<float><<<T, AP_THREADS, 0, stream>>>(proj, ld, (float*)q_out, H, G, D, Dv, rot, interleaved, q_w,
                                                                           k_w, eps, cos_t, sin_t, positions, slots, (float*)k_pool,
-                                                                          (float*)v_pool, page, has_kv);
+                                                                          (float*)v_pool, page, has_kv, per_head);
     else if (dtype == TM_BF16)
         whole_norm_rope_store_kernel<bf16_t><<<T, AP_THREADS, 0, stream>>>(proj, ld, (bf16_t*)q_out, H, G, D, Dv, rot, interleaved,
                                                                            q_w, k_w, eps, cos_t, sin_t, positions, slots,
-                                                                           (bf16_t*)k_pool, (bf16_t*)v_pool, page, has_kv);
+                                                                           (bf16_t*)k_pool, (bf16_t*)v_pool, page, has_kv, per_head);
     else
         return TM_ERR_ARG;
     TM_CHECK_LAUNCH();

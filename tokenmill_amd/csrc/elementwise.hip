@@ -34,6 +34,33 @@ extern "C" int tm_embed_gather(const void* table, int dtype, const int* ids, flo
     return TM_OK;
 }
 
+// out[t] = table[ids[t]] * scale: a model that multiplies its embedding rows by a constant on their way into the stream (the
+// product in 32-bit)
+template <typename T>
+__global__ void embed_gather_scaled_kernel(const T* __restrict__ table, const int* __restrict__ ids, float* __restrict__ out,
+                                           int hidden, int vocab, float scale) {
+    const int t = blockIdx.x;
+    int id = ids[t];
+    id = id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);       // the host rejects such ids; never read outside
+    const T* row = table + (size_t)id * hidden;
+    float* o = out + (size_t)t * hidden;
+    for (int c = threadIdx.x; c < hidden; c += blockDim.x) o[c] = Elem<T>::load(row + c) * scale;
+}
+
+extern "C" int tm_embed_gather_scaled(const void* table, int dtype, const int* ids, float* out, int T, int hidden, int vocab,
+                                      float scale, hipStream_t stream) {
+    if (T <= 0) return TM_OK;
+    if (hidden <= 0 || vocab <= 0 || !table || !ids || !out) return TM_ERR_ARG;
+    if (dtype == TM_F32)
+        embed_gather_scaled_kernel<float><<<T, 256, 0, stream>>>((const float*)table, ids, out, hidden, vocab, scale);
+    else if (dtype == TM_BF16)
+        embed_gather_scaled_kernel<bf16_t><<<T, 256, 0, stream>>>((const bf16_t*)table, ids, out, hidden, vocab, scale);
+    else
+        return TM_ERR_ARG;
+    TM_CHECK_LAUNCH();
+    return TM_OK;
+}
+
 // ------------------------------------------------------------------------------------------
 // embedding rows plus learned position rows -> 32-bit residual stream: out[t] = table[ids[t]] + places[positions[t]]
 // (the sum in 32-bit; no scaling of either)
@@ -474,6 +501,35 @@ static int launch_activation(const void* in, void* out, int dtype, long long n, 
         activation_kernel<float, ACT><<<blocks, 256, 0, stream>>>((const float*)in, (float*)out, (size_t)n);
     else if (dtype == TM_BF16)
         activation_kernel<bf16_t, ACT><<<blocks, 256, 0, stream>>>((const bf16_t*)in, (bf16_t*)out, (size_t)n);
+    else
+        return TM_ERR_ARG;
+    TM_CHECK_LAUNCH();
+    return TM_OK;
+}
+
+// out[t, i] = gelu_tanh(gu[t, i]) * gu[t, I + i]: the gated feed-forward's activation with the tanh form of GELU on the gate,
+// computed in 32-bit and rounded once; gu [T, 2I] (gate columns, then up columns).
+template <typename T>
+__global__ void gelu_mul_kernel(const T* __restrict__ gu, T* __restrict__ out, int I, size_t total) {
+    for (size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += (size_t)gridDim.x * blockDim.x) {
+        const size_t t = idx / I;
+        const int i = (int)(idx - t * I);
+        const float g = Elem<T>::load(gu + t * 2 * I + i);
+        const float u = Elem<T>::load(gu + t * 2 * I + I + i);
+        Elem<T>::store(out + idx, gelu_tanh_f32(g) * u);
+    }
+}
+
+extern "C" int tm_gelu_mul(const void* gu, void* out, int dtype, int T, int I, hipStream_t stream) {
+    if (T <= 0) return TM_OK;
+    if (I <= 0 || !gu || !out) return TM_ERR_ARG;
+    const size_t total = (size_t)T * I;
+    const size_t want = (total + 255) / 256;
+    const int blocks = (int)(want < 16384 ? want : 16384);
+    if (dtype == TM_F32)
+        gelu_mul_kernel<float><<<blocks, 256, 0, stream>>>((const float*)gu, (float*)out, I, total);
+    else if (dtype == TM_BF16)
+        gelu_mul_kernel<bf16_t><<<blocks, 256, 0, stream>>>((const bf16_t*)gu, (bf16_t*)out, I, total);
     else
         return TM_ERR_ARG;
     TM_CHECK_LAUNCH();

@@ -22,7 +22,7 @@ __global__ __launch_bounds__(256) void grouped_mfma_kernel(const bf16_t* __restr
                                                            const int* __restrict__ row_src, int src_div,
                                                            const bf16_t* __restrict__ W, void* __restrict__ Cv, int ldc, int c_off,
                                                            const float* __restrict__ gate, int ldg, const int* __restrict__ tiles,
-                                                           const int* __restrict__ n_tiles, int T, int K, int N, int tail, int rot,
+                                                           const int* __restrict__ n_tiles, int T, int K, int N, int tail, int rot_,
                                                            const float* __restrict__ cos_t, const float* __restrict__ sin_t,
                                                            const int* __restrict__ positions) {
     constexpr int BM = RT * 16;
@@ -117,19 +117,22 @@ __global__ __launch_bounds__(256) void grouped_mfma_kernel(const bf16_t* __restr
         }
         __syncthreads();
     }
-    // heads: the `tail` channels that follow a head's K input channels go behind its N output channels, their first `rot`
-    // rotated in pairs (2i, 2i + 1) by the row's position (the rotated part of a query head beside its part on the latent)
+    // heads: the `tail` channels that follow a head's K input channels go behind its N output channels, their first |rot_|
+    // rotated in pairs (2i, 2i + 1), or (i, i + |rot_| / 2) where rot_ < 0, by the row's position (the rotated part of a query
+    // head beside its part on the latent)
     if (MODE == GM_STORE && tail > 0 && blockIdx.y == 0) {
+        const int rot = rot_ < 0 ? -rot_ : rot_;
         const int half = rot / 2, rest = tail - rot;
         for (int idx = threadIdx.x; idx < rows * half; idx += 256) {
             const int row = row0 + idx / half, c = idx % half;
-            const bf16_t* sp = A + (size_t)row * lda + (size_t)group * a_off + K + 2 * c;
-            bf16_t* dp = (bf16_t*)Cv + (size_t)row * ldc + (size_t)group * c_off + N + 2 * c;
+            const int c1 = rot_ < 0 ? c : 2 * c, c2 = rot_ < 0 ? c + half : 2 * c + 1;
+            const bf16_t* sp = A + (size_t)row * lda + (size_t)group * a_off + K;
+            bf16_t* dp = (bf16_t*)Cv + (size_t)row * ldc + (size_t)group * c_off + N;
             const size_t at = (size_t)positions[row] * half + c;
             float a, b;
-            rotate_pair(bf16_to_f32(sp[0]), bf16_to_f32(sp[1]), cos_t[at], sin_t[at], a, b);
-            dp[0] = f32_to_bf16(a);
-            dp[1] = f32_to_bf16(b);
+            rotate_pair(bf16_to_f32(sp[c1]), bf16_to_f32(sp[c2]), cos_t[at], sin_t[at], a, b);
+            dp[c1] = f32_to_bf16(a);
+            dp[c2] = f32_to_bf16(b);
         }
         for (int idx = threadIdx.x; idx < rows * rest; idx += 256) {
             const int row = row0 + idx / rest, c = rot + idx % rest;
@@ -173,10 +176,10 @@ extern "C" int tm_heads_matmul_mfma_takes(const void* A, int lda, int a_off, con
 
 // C[t, h * c_off + n] = sum_k A[t, h * a_off + k] * W[h][n][k] (W [H, N, K]), times sigmoid(gate[t * ldg + h]) if gate.
 // tail > 0: also C[t, h * c_off + N + c] = A[t, h * a_off + K + c] for c < tail, the first `rot` of them rotated in pairs
-// (2i, 2i + 1) by positions[t] (cos_t, sin_t [positions, rot / 2]).
+// (2i, 2i + 1), or (i, i + rot / 2) with half_pairs, by positions[t] (cos_t, sin_t [positions, rot / 2]).
 extern "C" int tm_heads_matmul_mfma(const void* A, int lda, int a_off, const void* W, void* C, int ldc, int c_off, const float* gate,
                                     int ldg, int T, int H, int K, int N, int tail, int rot, const float* cos_t, const float* sin_t,
-                                    const int* positions, hipStream_t stream) {
+                                    const int* positions, int half_pairs, hipStream_t stream) {
     if (!A || !W || !C || T < 0 || H <= 0 || H > 65535 || K <= 0 || N <= 0 || tail < 0 || rot < 0 || rot > tail || rot % 2 ||
         a_off < K + tail || c_off < N + tail || !tm_heads_matmul_mfma_takes(A, lda, a_off, W, K) || (gate && ldg < H) ||
         (rot && (!cos_t || !sin_t || !positions)))
@@ -185,7 +188,8 @@ extern "C" int tm_heads_matmul_mfma(const void* A, int lda, int a_off, const voi
     dim3 grid((T + 63) / 64, (N + GM_BN - 1) / GM_BN, H);
     if (grid.y > 65535) return TM_ERR_ARG;
     grouped_mfma_kernel<4, GM_STORE><<<grid, 256, 0, stream>>>((const bf16_t*)A, lda, a_off, nullptr, 1, (const bf16_t*)W, C, ldc, c_off,
-                                                               gate, ldg, nullptr, nullptr, T, K, N, tail, rot, cos_t, sin_t, positions);
+                                                               gate, ldg, nullptr, nullptr, T, K, N, tail, half_pairs ? -rot : rot, cos_t, sin_t,
+                                                               positions);
     TM_CHECK_LAUNCH();
     return TM_OK;
 }

@@ -9,8 +9,10 @@
 //   tm_rotate_heads     dst[t, h, :Dr] = rotate(src[t, h, :Dr])                    the rotated part of every query head
 //   tm_attn_latent      out[t, h, :Lk] = softmax_j(scale * qa[t, h] . row[j]) . row[j, :Lk]   over the window's rows
 //
-// The rotation pairs channels (2i, 2i + 1), i < rot / 2, by the angle position * f_i (cos and sin from a 32-bit table
-// [positions, rot / 2]); channels from rot on pass unchanged. Norm statistics, scores, softmax and all sums are 32-bit.
+// The rotation pairs channels (2i, 2i + 1), i < rot / 2, or with `half_pairs` channels (i, i + rot / 2), by the angle
+// position * f_i (cos and sin from a 32-bit table [positions, rot / 2]); channels from rot on pass unchanged. Norm
+// statistics, scores, softmax and all sums are 32-bit. A softmax may have a sink: one more term exp(sink[h]) in the
+// denominator of head h, with no row behind it (sink null: none).
 #include "common.h"
 #include "api.h"
 
@@ -22,7 +24,7 @@ __global__ __launch_bounds__(LP_THREADS) void latent_prepare_kernel(const float*
                                                                     const float* __restrict__ wk, float eps,
                                                                     const float* __restrict__ cos_t, const float* __restrict__ sin_t,
                                                                     const int* __restrict__ positions, const int* __restrict__ slots,
-                                                                    T* __restrict__ cq, T* __restrict__ pool) {
+                                                                    T* __restrict__ cq, T* __restrict__ pool, int half_pairs) {
     __shared__ float red[LP_THREADS / TM_WAVE];
     const int t = blockIdx.x;
     const float* row = low + (size_t)t * ld;
@@ -33,8 +35,9 @@ __global__ __launch_bounds__(LP_THREADS) void latent_prepare_kernel(const float*
         const float inv = 1.0f / sqrtf(block_sum<LP_THREADS>(sq, red) / (float)Lq + eps);
         for (int c = threadIdx.x; c < Lq; c += LP_THREADS) Elem<T>::store(cq + (size_t)t * Lq + c, row[c] * inv * wq[c]);
     }
-    const float invk = 1.0f / sqrtf(block_sum<LP_THREADS>(sk, red) / (float)Lk + eps);
     const int slot = slots ? slots[t] : -1;
+    if (Lk == 0 || !slots) return;                            // a layer without a latent of its own: block-uniform
+    const float invk = 1.0f / sqrtf(block_sum<LP_THREADS>(sk, red) / (float)Lk + eps);
     if (slot < 0) return;
     T* dst = pool + (size_t)slot * (Lk + Dr);
     for (int c = threadIdx.x; c < Lk; c += LP_THREADS) Elem<T>::store(dst + c, row[Lq + c] * invk * wk[c]);
@@ -43,27 +46,29 @@ __global__ __launch_bounds__(LP_THREADS) void latent_prepare_kernel(const float*
     const int p = rot ? positions[t] : 0;
     for (int i = threadIdx.x; i < half; i += LP_THREADS) {
         float a, b;
-        rotate_pair(kr[2 * i], kr[2 * i + 1], cos_t[(size_t)p * half + i], sin_t[(size_t)p * half + i], a, b);
-        Elem<T>::store(dst + Lk + 2 * i, a);
-        Elem<T>::store(dst + Lk + 2 * i + 1, b);
+        const int i1 = half_pairs ? i : 2 * i, i2 = half_pairs ? i + half : 2 * i + 1;
+        rotate_pair(kr[i1], kr[i2], cos_t[(size_t)p * half + i], sin_t[(size_t)p * half + i], a, b);
+        Elem<T>::store(dst + Lk + i1, a);
+        Elem<T>::store(dst + Lk + i2, b);
     }
     for (int c = rot + threadIdx.x; c < Dr; c += LP_THREADS) Elem<T>::store(dst + Lk + c, kr[c]);
 }
 
 extern "C" int tm_latent_prepare(const float* low, int ld, int Lq, int Lk, int Dr, int rot, const float* wq, const float* wk,
                                  float eps, const float* cos_t, const float* sin_t, const int* positions, const int* slots,
-                                 void* cq, void* pool, int dtype, int T, hipStream_t stream) {
-    if (!low || Lq < 0 || Lk <= 0 || Dr < 0 || rot < 0 || rot > Dr || rot % 2 || ld < Lq + Lk + Dr || !wk || (Lq && (!wq || !cq)) ||
+                                 void* cq, void* pool, int dtype, int T, int half_pairs, hipStream_t stream) {
+    if (!low || Lq < 0 || Lk < 0 || Lq + Lk <= 0 || Dr < 0 || rot < 0 || rot > Dr || rot % 2 || ld < Lq + Lk + Dr || (Lk && !wk) ||
+        (!Lk && (slots || Dr)) || (Lq && (!wq || !cq)) ||
         (rot && (!cos_t || !sin_t || !positions)) || (slots && !pool) || !(eps > 0.f) || T < 0)
         return TM_ERR_ARG;
     if (dtype != TM_F32 && dtype != TM_BF16) return TM_ERR_ARG;
     if (T == 0) return TM_OK;
     if (dtype == TM_F32)
         latent_prepare_kernel<float><<<T, LP_THREADS, 0, stream>>>(low, ld, Lq, Lk, Dr, rot, wq, wk, eps, cos_t, sin_t, positions,
-                                                                   slots, (float*)cq, (float*)pool);
+                                                                   slots, (float*)cq, (float*)pool, half_pairs);
     else
         latent_prepare_kernel<bf16_t><<<T, LP_THREADS, 0, stream>>>(low, ld, Lq, Lk, Dr, rot, wq, wk, eps, cos_t, sin_t, positions,
-                                                                    slots, (bf16_t*)cq, (bf16_t*)pool);
+                                                                    slots, (bf16_t*)cq, (bf16_t*)pool, half_pairs);
     TM_CHECK_LAUNCH();
     return TM_OK;
 }
@@ -145,7 +150,7 @@ template <typename T>
 __global__ __launch_bounds__(256) void rotate_heads_kernel(const T* __restrict__ src, int lds_, int s_head, T* __restrict__ dst,
                                                            int ldd, int d_head, int H, int Dr, int rot,
                                                            const float* __restrict__ cos_t, const float* __restrict__ sin_t,
-                                                           const int* __restrict__ positions) {
+                                                           const int* __restrict__ positions, int half_pairs) {
     const int t = blockIdx.x;
     const int half = rot / 2;
     const int p = rot ? positions[t] : 0;
@@ -154,9 +159,10 @@ __global__ __launch_bounds__(256) void rotate_heads_kernel(const T* __restrict__
         const T* s = src + (size_t)t * lds_ + (size_t)h * s_head;
         T* d = dst + (size_t)t * ldd + (size_t)h * d_head;
         float a, b;
-        rotate_pair(Elem<T>::load(s + 2 * c), Elem<T>::load(s + 2 * c + 1), cos_t[(size_t)p * half + c], sin_t[(size_t)p * half + c], a, b);
-        Elem<T>::store(d + 2 * c, a);
-        Elem<T>::store(d + 2 * c + 1, b);
+        const int c1 = half_pairs ? c : 2 * c, c2 = half_pairs ? c + half : 2 * c + 1;
+        rotate_pair(Elem<T>::load(s + c1), Elem<T>::load(s + c2), cos_t[(size_t)p * half + c], sin_t[(size_t)p * half + c], a, b);
+        Elem<T>::store(d + c1, a);
+        Elem<T>::store(d + c2, b);
     }
     const int rest = Dr - rot;
     for (int i = threadIdx.x; i < H * rest; i += 256) {
@@ -166,7 +172,8 @@ __global__ __launch_bounds__(256) void rotate_heads_kernel(const T* __restrict__
 }
 
 extern "C" int tm_rotate_heads(const void* src, int ld_src, int src_head, void* dst, int ld_dst, int dst_head, int T, int H, int Dr,
-                               int rot, const float* cos_t, const float* sin_t, const int* positions, int dtype, hipStream_t stream) {
+                               int rot, const float* cos_t, const float* sin_t, const int* positions, int dtype, int half_pairs,
+                               hipStream_t stream) {
     if (!src || !dst || T < 0 || H <= 0 || Dr < 0 || rot < 0 || rot > Dr || rot % 2 || src_head < Dr || dst_head < Dr ||
         (rot && (!cos_t || !sin_t || !positions)))
         return TM_ERR_ARG;
@@ -174,10 +181,10 @@ extern "C" int tm_rotate_heads(const void* src, int ld_src, int src_head, void* 
     if (T == 0 || Dr == 0) return TM_OK;
     if (dtype == TM_F32)
         rotate_heads_kernel<float><<<T, 256, 0, stream>>>((const float*)src, ld_src, src_head, (float*)dst, ld_dst, dst_head, H, Dr, rot,
-                                                          cos_t, sin_t, positions);
+                                                          cos_t, sin_t, positions, half_pairs);
     else
         rotate_heads_kernel<bf16_t><<<T, 256, 0, stream>>>((const bf16_t*)src, ld_src, src_head, (bf16_t*)dst, ld_dst, dst_head, H, Dr,
-                                                           rot, cos_t, sin_t, positions);
+                                                           rot, cos_t, sin_t, positions, half_pairs);
     TM_CHECK_LAUNCH();
     return TM_OK;
 }
@@ -204,7 +211,8 @@ __global__ __launch_bounds__(AL_WAVES * TM_WAVE) void attn_latent_kernel(const T
                                                                          const int* __restrict__ block_tables, int table_width,
                                                                          const int* __restrict__ seq_of_token,
                                                                          const int* __restrict__ positions, int T_tokens, int H,
-                                                                         int Lk, int Dk, int page, float scale, int window) {
+                                                                         int Lk, int Dk, int page, float scale, int window,
+                                                                         const float* __restrict__ sink) {
     __shared__ float q_s[AL_WAVES][AL_MAX_DK];
     __shared__ float p_s[AL_WAVES][TM_WAVE];
     __shared__ int slot_s[AL_WAVES][TM_WAVE];
@@ -257,6 +265,7 @@ __global__ __launch_bounds__(AL_WAVES * TM_WAVE) void attn_latent_kernel(const T
         }
         wave_lds_sync();
     }
+    if (sink) l += __expf(sink[h] - m);                      // the sink: a term of the denominator without a row
     const float inv = 1.0f / l;
     T* o = out + (size_t)t * out_stride + (size_t)h * Lk;
 #pragma unroll
@@ -268,7 +277,7 @@ __global__ __launch_bounds__(AL_WAVES * TM_WAVE) void attn_latent_kernel(const T
 
 extern "C" int tm_attn_latent(const void* qa, int q_stride, void* out, int out_stride, const void* pool, const int* block_tables,
                               int table_width, const int* seq_of_token, const int* positions, int T, int H, int Lk, int Dk, int page,
-                              float scale, int window, int dtype, hipStream_t stream) {
+                              float scale, int window, const float* sink, int dtype, hipStream_t stream) {
     if (!qa || !out || !pool || !block_tables || !seq_of_token || !positions || T < 0 || H <= 0 || Lk <= 0 || Lk > Dk ||
         Dk > AL_MAX_DK || Lk > AL_MAX_ACC * TM_WAVE || page <= 0 || window < 0 || table_width <= 0 ||
         (long long)q_stride < (long long)H * Dk || (long long)out_stride < (long long)H * Lk)
@@ -281,11 +290,11 @@ extern "C" int tm_attn_latent(const void* qa, int q_stride, void* out, int out_s
     if (dtype == TM_F32)
         attn_latent_kernel<float><<<(unsigned)blocks, AL_WAVES * TM_WAVE, 0, stream>>>(
             (const float*)qa, q_stride, (float*)out, out_stride, (const float*)pool, block_tables, table_width, seq_of_token,
-            positions, T, H, Lk, Dk, page, scale, window);
+            positions, T, H, Lk, Dk, page, scale, window, sink);
     else
         attn_latent_kernel<bf16_t><<<(unsigned)blocks, AL_WAVES * TM_WAVE, 0, stream>>>(
             (const bf16_t*)qa, q_stride, (bf16_t*)out, out_stride, (const bf16_t*)pool, block_tables, table_width, seq_of_token,
-            positions, T, H, Lk, Dk, page, scale, window);
+            positions, T, H, Lk, Dk, page, scale, window, sink);
     TM_CHECK_LAUNCH();
     return TM_OK;
 }

@@ -32,7 +32,8 @@ __global__ __launch_bounds__(64 * WAVES) void attn_latent_mfma_kernel(
     const bf16_t* __restrict__ qa, int q_stride, bf16_t* __restrict__ out, int out_stride, const bf16_t* __restrict__ pool,
     const int* __restrict__ block_tables, int table_width, const int* __restrict__ tiles, int head_groups,
     const int* __restrict__ seq_of_token, const int* __restrict__ positions, int first_single, float* __restrict__ part_o,
-    float* __restrict__ part_ml, int n_chunks, int chunk_runs, int H, int Lk, int Dk, int page, float scale_log2, int window) {
+    float* __restrict__ part_ml, int n_chunks, int chunk_runs, int H, int Lk, int Dk, int page, float scale_log2, int window,
+    const float* __restrict__ sink) {
     extern __shared__ __align__(16) unsigned char lds_raw[];
     const int DKP = (Dk + 31) / 32 * 32, ndc = DKP / 32;
     const int ks_stride = DKP + LM_PAD;
@@ -203,6 +204,8 @@ __global__ __launch_bounds__(64 * WAVES) void attn_latent_mfma_kernel(
         }
         return;
     }
+    // the sink of the pair's head: one more term of the denominator, with no row behind it (m is a power of two's exponent)
+    if (sink) total += __builtin_amdgcn_exp2f(sink[head] * 1.4426950408889634f - m);
     const float inv = 1.0f / total;
     bf16_t* dst = out + (size_t)token * out_stride + (size_t)head * Lk;
 #pragma unroll
@@ -213,10 +216,11 @@ __global__ __launch_bounds__(64 * WAVES) void attn_latent_mfma_kernel(
 }
 
 // out[token, head] = sum_y part_o[y] 2^(m_y - M) / sum_y l_y 2^(m_y - M), M = max_y m_y, chunks y in their order; a chunk
-// without a visible row (m = -inf, zeros in part_o) weighs nothing.
+// without a visible row (m = -inf, zeros in part_o) weighs nothing. With a sink, L also holds 2^(sink[h] log2 e - M) and M is
+// at least the sink's exponent.
 __global__ __launch_bounds__(128) void attn_latent_merge_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
                                                                 bf16_t* __restrict__ out, int out_stride, int first_single, int H,
-                                                                int Lk, int n_chunks) {
+                                                                int Lk, int n_chunks, const float* __restrict__ sink) {
     extern __shared__ float w_s[];                                        // a chunk's weight 2^(m_y - M) / L
     const int pair = blockIdx.x, t = pair / H, h = pair % H;
     const float* ml = part_ml + (size_t)pair * n_chunks * 2;
@@ -224,7 +228,9 @@ __global__ __launch_bounds__(128) void attn_latent_merge_kernel(const float* __r
         float M = -INFINITY;
         for (int y = threadIdx.x; y < n_chunks; y += TM_WAVE) M = fmaxf(M, ml[2 * y]);
         M = wave_max(M);
-        float L = 0.f;
+        const float sk = sink ? sink[h] * 1.4426950408889634f : -INFINITY;
+        M = fmaxf(M, sk);
+        float L = sink ? __builtin_amdgcn_exp2f(sk - M) : 0.f;
         for (int y0 = 0; y0 < n_chunks; y0 += TM_WAVE) {                  // the chunks' sums in their order, 64 at a time
             const int y = y0 + threadIdx.x;
             const float e = (y < n_chunks && ml[2 * y] != -INFINITY) ? ml[2 * y + 1] * __builtin_amdgcn_exp2f(ml[2 * y] - M) : 0.f;
@@ -272,7 +278,7 @@ extern "C" int tm_attn_latent_chunks(int most_rows, int chunk_runs) {
 struct LmArgs {
     const bf16_t* qa; int q_stride; bf16_t* out; int out_stride; const bf16_t* pool; const int* block_tables; int table_width;
     const int* tiles; int head_groups; const int* seq_of_token; const int* positions; int first_single; float* part_o;
-    float* part_ml; int n_chunks; int chunk_runs; int H, Lk, Dk, page; float scale_log2; int window;
+    float* part_ml; int n_chunks; int chunk_runs; int H, Lk, Dk, page; float scale_log2; int window; const float* sink;
 };
 
 template <int WAVES, int NDT, int NDC, int SPLIT>
@@ -286,7 +292,8 @@ static int lm_launch(dim3 grid, size_t lds, hipStream_t stream, const LmArgs& a)
     }
     kernel<<<grid, 64 * WAVES, lds, stream>>>(a.qa, a.q_stride, a.out, a.out_stride, a.pool, a.block_tables, a.table_width, a.tiles,
                                               a.head_groups, a.seq_of_token, a.positions, a.first_single, a.part_o, a.part_ml,
-                                              a.n_chunks, a.chunk_runs, a.H, a.Lk, a.Dk, a.page, a.scale_log2, a.window);
+                                              a.n_chunks, a.chunk_runs, a.H, a.Lk, a.Dk, a.page, a.scale_log2, a.window,
+                                              a.part_o ? nullptr : a.sink);      // a chunk's share meets the sink in the merge, once
     return TM_OK;
 }
 
@@ -311,7 +318,7 @@ extern "C" int tm_attn_latent_mfma(const void* qa, int q_stride, void* out, int 
                                    const int* block_tables, int table_width, const int* tiles, int n_tiles,
                                    const int* seq_of_token, const int* positions, int first_single, int n_single, float* part_o,
                                    float* part_ml, int n_chunks, int chunk_runs, int H, int Lk, int Dk, int page, float scale,
-                                   int window, hipStream_t stream) {
+                                   int window, const float* sink, hipStream_t stream) {
     if ((n_tiles > 0) == (n_single > 0)) return (n_tiles == 0 && n_single == 0) ? TM_OK : TM_ERR_ARG;
     if (!qa || !out || !pool || !block_tables || H <= 0 || page <= 0 || window < 0 || table_width <= 0 ||
         !tm_attn_latent_mfma_takes(Lk, Dk, q_stride, out_stride) || ((uintptr_t)qa % 16) || ((uintptr_t)out % 8) ||
@@ -322,7 +329,7 @@ extern "C" int tm_attn_latent_mfma(const void* qa, int q_stride, void* out, int 
         return TM_ERR_ARG;
     LmArgs a{(const bf16_t*)qa, q_stride, (bf16_t*)out, out_stride, (const bf16_t*)pool, block_tables, table_width,
              n_tiles > 0 ? tiles : nullptr, 1, seq_of_token, positions, first_single, nullptr, nullptr, n_chunks, chunk_runs,
-             H, Lk, Dk, page, scale * 1.4426950408889634f, window};
+             H, Lk, Dk, page, scale * 1.4426950408889634f, window, sink};
     const size_t lds = lm_lds_bytes(Lk, Dk);
     int rc;
     if (n_tiles > 0) {
@@ -340,7 +347,7 @@ extern "C" int tm_attn_latent_mfma(const void* qa, int q_stride, void* out, int 
         if (rc == TM_OK) {
             TM_CHECK_LAUNCH();
             attn_latent_merge_kernel<<<n_single * H, 128, (size_t)n_chunks * sizeof(float), stream>>>(part_o, part_ml, (bf16_t*)out, out_stride, first_single, H, Lk,
-                                                                       n_chunks);
+                                                                       n_chunks, sink);
         }
     }
     if (rc != TM_OK) return rc;

@@ -3,7 +3,8 @@
 //
 //   pair p = (token t = p / top, choice k = p % top) goes to expert e(p) = table[id[t] * top + k]  (ids null: table[p])
 //   tm_moe_router    z [T, E] (32-bit router outputs) -> s = softmax(z); the `top` largest of s + correction are chosen
-//                    (ties: the lower index), chosen[t, k] in descending order, weight[t, k] = s / (sum of the chosen s + 1e-20)
+//                    (ties: the lower index), chosen[t, k] in descending order, weight[t, k] = s / (sum of the chosen s + 1e-20);
+//                    with `over_chosen` the `top` largest z are chosen and the weights are the softmax over the chosen z only
 //   tm_moe_route     sorts the pairs by expert: slot_pair[slot] = p, pair_slot[p] = slot, and cuts every expert's run of
 //                    slots into tiles of `tile_rows` rows: tiles[i] = (expert, first slot, rows), n_tiles[0] = their number
 //   tm_moe_gate_up   act[slot] = silu(x[t] . Wg[e]^T) * (x[t] . Wu[e]^T)          W [E, 2F, K]: gate rows, then up rows
@@ -244,7 +245,8 @@ extern "C" int tm_moe_combine(const float* part, const int* pair_slot, void* y, 
 // Everything is 32-bit.
 template <int RT_MAX_PER_LANE>
 __global__ __launch_bounds__(TM_WAVE) void moe_router_kernel(const float* __restrict__ z, int ldz, const float* __restrict__ correction,
-                                                             int E, int top, int* __restrict__ chosen, float* __restrict__ weight) {
+                                                             int E, int top, int* __restrict__ chosen, float* __restrict__ weight,
+                                                             int over_chosen) {
     const int t = blockIdx.x, lane = threadIdx.x;
     const float* zr = z + (size_t)t * ldz;
     float s[RT_MAX_PER_LANE], c[RT_MAX_PER_LANE];
@@ -260,15 +262,18 @@ __global__ __launch_bounds__(TM_WAVE) void moe_router_kernel(const float* __rest
 #pragma unroll
     for (int i = 0; i < RT_MAX_PER_LANE; ++i) {
         const int e = lane + i * TM_WAVE;
-        s[i] = e < E ? expf(s[i] - m) : 0.f;
+        c[i] = s[i];                             // the output itself: what `over_chosen` ranks
+        s[i] = e < E ? expf(s[i] - m) : 0.f;     // m is the largest output, which is chosen first: these are the chosen ones' terms too
         sum += s[i];
     }
     sum = wave_sum(sum);
+    if (!over_chosen) {
 #pragma unroll
-    for (int i = 0; i < RT_MAX_PER_LANE; ++i) {
-        const int e = lane + i * TM_WAVE;
-        s[i] = s[i] / sum;
-        c[i] = e < E ? s[i] + (correction ? correction[e] : 0.f) : -INFINITY;
+        for (int i = 0; i < RT_MAX_PER_LANE; ++i) {
+            const int e = lane + i * TM_WAVE;
+            s[i] = s[i] / sum;
+            c[i] = e < E ? s[i] + (correction ? correction[e] : 0.f) : -INFINITY;
+        }
     }
     float total = 0.f;
     for (int k = 0; k < top; ++k) {
@@ -293,17 +298,18 @@ __global__ __launch_bounds__(TM_WAVE) void moe_router_kernel(const float* __rest
         }
     }
     __syncthreads();                         // lane 0's scores, seen by the lanes that scale them
-    const float inv = 1.f / (total + 1e-20f);
+    const float inv = over_chosen ? 1.f / total : 1.f / (total + 1e-20f);
     for (int k = lane; k < top; k += TM_WAVE) weight[(size_t)t * top + k] *= inv;
 }
 
 extern "C" int tm_moe_router(const float* z, int ldz, const float* correction, int T, int E, int top, int* chosen, float* weight,
-                             hipStream_t stream) {
+                             int over_chosen, hipStream_t stream) {
     if (!z || !chosen || !weight || T < 0 || E <= 0 || E > MOE_MAX_EXPERTS || top <= 0 || top > E || ldz < E) return TM_ERR_ARG;
     if (T == 0) return TM_OK;
-    if (E <= TM_WAVE) moe_router_kernel<1><<<T, TM_WAVE, 0, stream>>>(z, ldz, correction, E, top, chosen, weight);
-    else if (E <= 4 * TM_WAVE) moe_router_kernel<4><<<T, TM_WAVE, 0, stream>>>(z, ldz, correction, E, top, chosen, weight);
-    else moe_router_kernel<MOE_MAX_EXPERTS / TM_WAVE><<<T, TM_WAVE, 0, stream>>>(z, ldz, correction, E, top, chosen, weight);
+    if (over_chosen && correction) return TM_ERR_ARG;
+    if (E <= TM_WAVE) moe_router_kernel<1><<<T, TM_WAVE, 0, stream>>>(z, ldz, correction, E, top, chosen, weight, over_chosen);
+    else if (E <= 4 * TM_WAVE) moe_router_kernel<4><<<T, TM_WAVE, 0, stream>>>(z, ldz, correction, E, top, chosen, weight, over_chosen);
+    else moe_router_kernel<MOE_MAX_EXPERTS / TM_WAVE><<<T, TM_WAVE, 0, stream>>>(z, ldz, correction, E, top, chosen, weight, over_chosen);
     TM_CHECK_LAUNCH();
     return TM_OK;
 }

@@ -73,14 +73,18 @@ def _ints(t: torch.Tensor, n: int, name: str) -> None:
 
 # --------------------------------------------------------------------------------------------
 
-def embed_gather(table: torch.Tensor, ids: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
-    """out[t] = table[ids[t]] as 32-bit rows. table [V, hidden], ids int32 [T], out float32 [T, hidden]."""
+def embed_gather(table: torch.Tensor, ids: torch.Tensor, out: torch.Tensor, scale: float = 1.0) -> torch.Tensor:
+    """out[t] = table[ids[t]] * scale as 32-bit rows. table [V, hidden], ids int32 [T], out float32 [T, hidden]."""
     _gpu(table, ids, out)
     T = ids.numel()
     V, hidden = table.shape
     _need(table.is_contiguous() and out.is_contiguous(), "embed_gather: operands must be contiguous")
     _need(out.dtype == torch.float32 and tuple(out.shape) == (T, hidden), "embed_gather: out must be float32 [T, hidden]")
     _ints(ids, T, "ids")
+    if scale != 1.0:
+        _check(library().tm_embed_gather_scaled(_p(table), code(table.dtype), _p(ids), _p(out), c_int(T), c_int(hidden), c_int(V),
+                                                c_float(scale), _stream()), "embed_gather_scaled")
+        return out
     _check(library().tm_embed_gather(_p(table), code(table.dtype), _p(ids), _p(out), c_int(T), c_int(hidden),
                                      c_int(V), _stream()), "embed_gather")
     return out
@@ -144,6 +148,16 @@ def silu_mul(gu: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
     _need(two_i % 2 == 0 and tuple(out.shape) == (T, two_i // 2) and gu.is_contiguous() and out.is_contiguous()
           and gu.dtype == out.dtype, "silu_mul: gu [T, 2I] and out [T, I] of one type, contiguous")
     _check(library().tm_silu_mul(_p(gu), _p(out), code(gu.dtype), c_int(T), c_int(two_i // 2), _stream()), "silu_mul")
+    return out
+
+
+def gelu_mul(gu: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    """out[t, i] = gelu_tanh(gu[t, i]) * gu[t, I + i], computed in 32-bit; gu [T, 2I], out [T, I]."""
+    _gpu(gu, out)
+    T, two_i = gu.shape
+    _need(two_i % 2 == 0 and tuple(out.shape) == (T, two_i // 2) and gu.is_contiguous() and out.is_contiguous()
+          and gu.dtype == out.dtype, "gelu_mul: gu [T, 2I] and out [T, I] of one type, contiguous")
+    _check(library().tm_gelu_mul(_p(gu), _p(out), code(gu.dtype), c_int(T), c_int(two_i // 2), _stream()), "gelu_mul")
     return out
 
 
@@ -1398,24 +1412,29 @@ def _angles(cos, sin, rot: int, positions, T: int, who: str) -> None:
         _ints(positions, T, "positions")
 
 
-def latent_prepare(low: torch.Tensor, Lq: int, Lk: int, Dr: int, wq: torch.Tensor | None, wk: torch.Tensor, eps: float,
+def latent_prepare(low: torch.Tensor, Lq: int, Lk: int, Dr: int, wq: torch.Tensor | None, wk: torch.Tensor | None, eps: float,
                    cos: torch.Tensor | None, sin: torch.Tensor | None, positions: torch.Tensor | None, slots: torch.Tensor | None,
-                   cq: torch.Tensor | None, pool: torch.Tensor | None) -> None:
+                   cq: torch.Tensor | None, pool: torch.Tensor | None, half_pairs: bool = False) -> None:
     """low float32 [T, >= Lq + Lk + Dr] = [query latent | key/value latent | shared key]: cq [T, Lq] = rms_norm(query latent) * wq;
     the cache row of token t (slot slots[t] of pool; < 0: not stored) = [rms_norm(latent) * wk | shared key with its first
-    2 * cos.shape[1] channels rotated in pairs (2i, 2i + 1) by the token's position]."""
+    2 * cos.shape[1] channels rotated in pairs (2i, 2i + 1), or (i, i + half) with ``half_pairs``, by the token's position].
+    Lk = 0 (with Dr = 0 and no slots): a layer that has only queries of its own."""
     _gpu(low, wq, wk, cos, sin, positions, slots, cq, pool)
     T = low.shape[0]
     _need(low.dtype == torch.float32 and low.dim() == 2 and low.stride(1) == 1 and low.shape[1] >= Lq + Lk + Dr,
           f"latent_prepare: low is float32 [T, >= {Lq + Lk + Dr}]")
-    _need(wk.dtype == torch.float32 and tuple(wk.shape) == (Lk,) and wk.is_contiguous(), f"latent_prepare: wk is float32 [{Lk}]")
+    if Lk:
+        _need(wk is not None and wk.dtype == torch.float32 and tuple(wk.shape) == (Lk,) and wk.is_contiguous(),
+              f"latent_prepare: wk is float32 [{Lk}]")
+    else:
+        _need(Dr == 0 and slots is None and Lq > 0, "latent_prepare: without a key/value latent there is nothing to store")
     dt = None
     if Lq:
         _need(wq is not None and wq.dtype == torch.float32 and tuple(wq.shape) == (Lq,) and wq.is_contiguous(),
               f"latent_prepare: wq is float32 [{Lq}]")
         _need(cq is not None and tuple(cq.shape) == (T, Lq) and cq.is_contiguous(), f"latent_prepare: cq is contiguous [T, {Lq}]")
         dt = cq.dtype
-    rot = 2 * cos.shape[1] if cos is not None else 0
+    rot = 2 * cos.shape[1] if (cos is not None and Dr) else 0
     _need(rot <= Dr, "latent_prepare: more rotated channels than the shared key has")
     _angles(cos, sin, rot, positions, T, "latent_prepare")
     if slots is not None:
@@ -1426,8 +1445,9 @@ def latent_prepare(low: torch.Tensor, Lq: int, Lk: int, Dr: int, wq: torch.Tenso
     _need(dt is not None, "latent_prepare: nothing to do")
     ld = low.stride(0) if T > 1 else max(low.stride(0), low.shape[1])
     _check(library().tm_latent_prepare(_p(low), c_int(ld), c_int(Lq), c_int(Lk), c_int(Dr), c_int(rot), _p(wq), _p(wk), c_float(eps),
-                                       _p(cos), _p(sin), _p(positions), _p(slots), _p(cq), _p(pool if slots is not None else None),
-                                       c_int(code(dt)), c_int(T), _stream()), "latent_prepare")
+                                       _p(cos if rot else None), _p(sin if rot else None), _p(positions if rot else None), _p(slots), _p(cq),
+                                       _p(pool if slots is not None else None), c_int(code(dt)), c_int(T), c_int(1 if half_pairs else 0),
+                                       _stream()), "latent_prepare")
 
 
 def heads_matmul(a: torch.Tensor, a_head: int, b: torch.Tensor, c: torch.Tensor, c_head: int,
@@ -1465,11 +1485,12 @@ def heads_matmul_mfma_takes(a: torch.Tensor, a_head: int, w: torch.Tensor) -> bo
 
 def heads_matmul_mfma(a: torch.Tensor, a_head: int, w: torch.Tensor, c: torch.Tensor, c_head: int,
                       gate: torch.Tensor | None = None, tail: int = 0, cos: torch.Tensor | None = None,
-                      sin: torch.Tensor | None = None, positions: torch.Tensor | None = None) -> torch.Tensor:
+                      sin: torch.Tensor | None = None, positions: torch.Tensor | None = None, half_pairs: bool = False) -> torch.Tensor:
     """``heads_matmul`` on the matrix unit, with the matrices given as w [H, N, K] (k contiguous): c[t, h * c_head + n] =
     sum_k a[t, h * a_head + k] * w[h, n, k], times sigmoid(gate[t, h]) if ``gate`` (float32 [T, >= H]). ``tail`` > 0: the
     ``tail`` channels behind a head's K input channels are copied behind its N output channels, the first 2 * cos.shape[1]
-    of them rotated in pairs (2i, 2i + 1) by the row's position (``rotate_heads`` in the same launch)."""
+    of them rotated in pairs (2i, 2i + 1), or (i, i + half) with ``half_pairs``, by the row's position (``rotate_heads`` in the
+    same launch)."""
     _gpu(a, w, c, gate)
     T = a.shape[0]
     H, N, K = w.shape
@@ -1492,13 +1513,13 @@ def heads_matmul_mfma(a: torch.Tensor, a_head: int, w: torch.Tensor, c: torch.Te
     ldc = c.stride(0) if T > 1 else max(c.stride(0), c.shape[1])
     _check(library().tm_heads_matmul_mfma(_p(a), c_int(lda), c_int(a_head), _p(w), _p(c), c_int(ldc), c_int(c_head), _p(gate),
                                           c_int(gate_stride), c_int(T), c_int(H), c_int(K), c_int(N), c_int(tail), c_int(rot),
-                                          _p(cos if rot else None), _p(sin if rot else None), _p(positions if rot else None), _stream()),
-           "heads_matmul_mfma")
+                                          _p(cos if rot else None), _p(sin if rot else None), _p(positions if rot else None),
+                                          c_int(1 if half_pairs else 0), _stream()), "heads_matmul_mfma")
     return c
 
 
 def rotate_heads(src: torch.Tensor, src_head: int, dst: torch.Tensor, dst_head: int, H: int, Dr: int, cos: torch.Tensor | None,
-                 sin: torch.Tensor | None, positions: torch.Tensor | None) -> None:
+                 sin: torch.Tensor | None, positions: torch.Tensor | None, half_pairs: bool = False) -> None:
     """dst[t, h * dst_head + c] = src[t, h * src_head + c] for c < Dr, the first 2 * cos.shape[1] channels of every head rotated in
     pairs (2i, 2i + 1) by the token's position. src and dst are views that start at the heads' first rotated channel."""
     _gpu(src, dst, cos, sin, positions)
@@ -1513,18 +1534,26 @@ def rotate_heads(src: torch.Tensor, src_head: int, dst: torch.Tensor, dst_head: 
     lds = src.stride(0) if T > 1 else max(src.stride(0), src.shape[1])
     ldd = dst.stride(0) if T > 1 else max(dst.stride(0), dst.shape[1])
     _check(library().tm_rotate_heads(_p(src), c_int(lds), c_int(src_head), _p(dst), c_int(ldd), c_int(dst_head), c_int(T), c_int(H),
-                                     c_int(Dr), c_int(rot), _p(cos), _p(sin), _p(positions), c_int(code(src.dtype)), _stream()),
-           "rotate_heads")
+                                     c_int(Dr), c_int(rot), _p(cos), _p(sin), _p(positions), c_int(code(src.dtype)),
+                                     c_int(1 if half_pairs else 0), _stream()), "rotate_heads")
 
 
 LATENT_MAX_ROW, LATENT_MAX_RANK = 704, 512
 
 
+def _check_sink(sink: torch.Tensor | None, H: int) -> None:
+    if sink is not None:
+        _need(sink.dtype == torch.float32 and tuple(sink.shape) == (H,) and sink.is_contiguous(), f"attention: sink is float32 [{H}]")
+
+
 def attn_latent(qa: torch.Tensor, out: torch.Tensor, pool: torch.Tensor, block_tables: torch.Tensor, seq_of_token: torch.Tensor,
-                positions: torch.Tensor, H: int, Lk: int, Dk: int, scale: float, window: int = 0) -> torch.Tensor:
+                positions: torch.Tensor, H: int, Lk: int, Dk: int, scale: float, window: int = 0,
+                sink: torch.Tensor | None = None) -> torch.Tensor:
     """out[t, h, :Lk] = sum_j softmax_j(scale * qa[t, h, :Dk] . row[j]) * row[j, :Lk] over the cached rows j of the token's
-    request with 0 <= position - j < window (0: every row up to the token's own). qa [T, H * Dk], out [T, H * Lk]."""
-    _gpu(qa, out, pool, block_tables, seq_of_token, positions)
+    request with 0 <= position - j < window (0: every row up to the token's own). qa [T, H * Dk], out [T, H * Lk]. ``sink``
+    (float32 [H]): one more term exp(sink[h]) in the softmax's denominator, with no row behind it."""
+    _gpu(qa, out, pool, block_tables, seq_of_token, positions, sink)
+    _check_sink(sink, H)
     T = qa.shape[0]
     _need(qa.is_contiguous() and tuple(qa.shape) == (T, H * Dk) and out.is_contiguous() and tuple(out.shape) == (T, H * Lk)
           and qa.dtype == out.dtype, f"attention(latent): qa [T, {H * Dk}] and out [T, {H * Lk}] contiguous, of one type")
@@ -1537,7 +1566,7 @@ def attn_latent(qa: torch.Tensor, out: torch.Tensor, pool: torch.Tensor, block_t
     _need(window >= 0, "attention(latent): window must be >= 0")
     _check(library().tm_attn_latent(_p(qa), c_int(H * Dk), _p(out), c_int(H * Lk), _p(pool), _p(block_tables), c_int(block_tables.shape[1]),
                                     _p(seq_of_token), _p(positions), c_int(T), c_int(H), c_int(Lk), c_int(Dk), c_int(page),
-                                    c_float(scale), c_int(window), c_int(code(qa.dtype)), _stream()), "attn_latent")
+                                    c_float(scale), c_int(window), _p(sink), c_int(code(qa.dtype)), _stream()), "attn_latent")
     return out
 
 
@@ -1548,13 +1577,15 @@ def attn_latent_mfma_takes(dtype, Lk: int, Dk: int, H: int) -> bool:
 
 def attn_latent_mfma(qa: torch.Tensor, out: torch.Tensor, pool: torch.Tensor, block_tables: torch.Tensor, tiles: torch.Tensor | None,
                      seq_of_token: torch.Tensor, positions: torch.Tensor, first_single: int, n_single: int, H: int, Lk: int, Dk: int,
-                     scale: float, window: int = 0, most_context: int = 0, bound: int = 0) -> torch.Tensor:
+                     scale: float, window: int = 0, most_context: int = 0, bound: int = 0,
+                     sink: torch.Tensor | None = None) -> torch.Tensor:
     """``attn_latent`` on the matrix unit for bfloat16: with ``tiles`` (int32 [n, 4]: request, first row, tokens, first position)
     the prompt portions of the step, tile by tile; with ``tiles`` None the ``n_single`` single tokens that start at row
     ``first_single``, none of which sits beyond position ``most_context`` - 1 (their visible rows are dealt in chunks to blocks
     of their own and merged in chunk order; ``bound``: the most rows the model lets any token see, its window or its longest
     context, which sets the chunks' size). Rows of qa / out that neither names are left alone."""
-    _gpu(qa, out, pool, block_tables, tiles, seq_of_token, positions)
+    _gpu(qa, out, pool, block_tables, tiles, seq_of_token, positions, sink)
+    _check_sink(sink, H)
     T = qa.shape[0]
     _need(qa.dtype == torch.bfloat16 and out.dtype == torch.bfloat16, "attention(latent, matrix unit): bfloat16 only")
     _need(qa.is_contiguous() and tuple(qa.shape) == (T, H * Dk) and out.is_contiguous() and tuple(out.shape) == (T, H * Lk),
@@ -1580,7 +1611,8 @@ def attn_latent_mfma(qa: torch.Tensor, out: torch.Tensor, pool: torch.Tensor, bl
     _check(library().tm_attn_latent_mfma(_p(qa), c_int(H * Dk), _p(out), c_int(H * Lk), _p(pool), _p(block_tables),
                                          c_int(block_tables.shape[1]), _p(tiles), c_int(n_tiles), _p(seq_of_token), _p(positions),
                                          c_int(first_single), c_int(n_single), _p(part_o), _p(part_ml), c_int(n_chunks), c_int(chunk_runs), c_int(H),
-                                         c_int(Lk), c_int(Dk), c_int(page), c_float(scale), c_int(window), _stream()), "attn_latent_mfma")
+                                         c_int(Lk), c_int(Dk), c_int(page), c_float(scale), c_int(window), _p(sink), _stream()),
+           "attn_latent_mfma")
     return out
 
 
@@ -1668,21 +1700,23 @@ def moe_experts(x: torch.Tensor, routed, w_gate_up: torch.Tensor, w_down: torch.
 def whole_norm_rope_store(proj: torch.Tensor, q_out: torch.Tensor, H: int, G: int, D: int, Dv: int, q_w: torch.Tensor | None,
                           k_w: torch.Tensor | None, eps: float, cos: torch.Tensor | None, sin: torch.Tensor | None, interleaved: bool,
                           positions: torch.Tensor | None, slots: torch.Tensor | None, k_pool: torch.Tensor | None,
-                          v_pool: torch.Tensor | None, has_kv: bool = True) -> torch.Tensor:
+                          v_pool: torch.Tensor | None, has_kv: bool = True, per_head: bool = False) -> torch.Tensor:
     """proj float32 [T, >= H*D (+ G*D + G*Dv)]: q (and k) are divided by the root mean square of the whole projection (all
     heads of a token at once) and multiplied by q_w [H*D] / k_w [G*D] (float32; None: no norm), the first 2 * cos.shape[1]
     channels of every head rotated by the token's position (pairs (j, j + rot/2), or (2j, 2j + 1) if ``interleaved``); q goes
     to q_out [T, H*D], k and v to the tokens' cache slots. ``has_kv`` False: the row holds no k and v (a layer that reads
-    another layer's cache)."""
+    another layer's cache). ``per_head``: every head of q and of k is normed by itself over its D channels, with weights [D] that
+    the heads share."""
     _gpu(proj, q_out, q_w, k_w, cos, sin, positions, slots, k_pool, v_pool)
     T = proj.shape[0]
     width = H * D + (G * (D + Dv) if has_kv else 0)
     _need(proj.dtype == torch.float32 and proj.dim() == 2 and proj.stride(1) == 1 and proj.shape[1] >= width,
           f"whole_norm_rope_store: proj is float32 [T, >= {width}]")
     _need(tuple(q_out.shape) == (T, H * D) and q_out.is_contiguous(), f"whole_norm_rope_store: q_out is contiguous [T, {H * D}]")
-    for w, n in ((q_w, H * D), (k_w, G * D)):
+    for w, n in ((q_w, D if per_head else H * D), (k_w, D if per_head else G * D)):
         if w is not None:
             _need(w.dtype == torch.float32 and tuple(w.shape) == (n,) and w.is_contiguous(), f"whole_norm_rope_store: a norm weight is float32 [{n}]")
+    _need(not per_head or H + G <= 1024, "whole_norm_rope_store: up to 1024 heads of q and k are normed by themselves")
     _need(not has_kv or (q_w is None) == (k_w is None), "whole_norm_rope_store: q and k are normed together or not at all")
     rot = 0
     if cos is not None:
@@ -1700,7 +1734,7 @@ def whole_norm_rope_store(proj: torch.Tensor, q_out: torch.Tensor, H: int, G: in
                                               c_int(D), c_int(Dv), c_int(rot), c_int(1 if interleaved else 0), _p(q_w), _p(k_w),
                                               c_float(eps), _p(cos), _p(sin), _p(positions), _p(slots if write else None),
                                               _p(k_pool if write else None), _p(v_pool if write else None), c_int(page),
-                                              c_int(1 if has_kv else 0), _stream()), "whole_norm_rope_store")
+                                              c_int(1 if has_kv else 0), c_int(1 if per_head else 0), _stream()), "whole_norm_rope_store")
     return q_out
 
 
@@ -1738,14 +1772,16 @@ def attn_paged_softmax(q: torch.Tensor, out: torch.Tensor, k_pool: torch.Tensor,
 
 # -------------------------------------------------------------------------------------------- experts by router
 
-def moe_router(z: torch.Tensor, experts: int, top: int, correction: torch.Tensor | None = None):
+def moe_router(z: torch.Tensor, experts: int, top: int, correction: torch.Tensor | None = None, over_chosen: bool = False):
     """z: float32 view [T, >= experts] (the router's outputs). s = softmax over the first ``experts`` columns; the ``top``
     largest of s + correction are chosen (descending; of equals the lower index). Returns (chosen int32 [T, top], weight
-    float32 [T, top] = the chosen experts' s divided by their sum + 1e-20)."""
+    float32 [T, top] = the chosen experts' s divided by their sum + 1e-20). ``over_chosen``: the ``top`` largest z themselves are
+    chosen and the weights are the softmax over the chosen z only (no correction)."""
     _gpu(z, correction)
     T = z.shape[0]
     _need(z.dtype == torch.float32 and z.dim() == 2 and z.stride(1) == 1 and z.shape[1] >= experts, f"moe_router: z is float32 [T, >= {experts}]")
     _need(0 < top <= experts <= MOE_MAX_EXPERTS, f"moe_router: {top} of {experts} experts (up to {MOE_MAX_EXPERTS})")
+    _need(not (over_chosen and correction is not None), "moe_router: a correction shifts a choice among softmax scores only")
     if correction is not None:
         _need(correction.dtype == torch.float32 and tuple(correction.shape) == (experts,) and correction.is_contiguous(),
               f"moe_router: correction is float32 [{experts}]")
@@ -1753,7 +1789,7 @@ def moe_router(z: torch.Tensor, experts: int, top: int, correction: torch.Tensor
     weight = torch.empty((T, top), dtype=torch.float32, device=z.device)
     ldz = z.stride(0) if T > 1 else max(z.stride(0), experts)
     _check(library().tm_moe_router(_p(z), c_int(ldz), _p(correction), c_int(T), c_int(experts), c_int(top), _p(chosen), _p(weight),
-                                   _stream()), "moe_router")
+                                   c_int(1 if over_chosen else 0), _stream()), "moe_router")
     return chosen, weight
 
 
@@ -1775,10 +1811,12 @@ def moe_route_chosen(chosen: torch.Tensor, experts: int, real: int, tile_rows: i
 
 
 def moe_experts_weighted(x: torch.Tensor, routed, weight: torch.Tensor, w_up: torch.Tensor | None, w_down: torch.Tensor | None, top: int,
-                         out: torch.Tensor, shared: torch.Tensor | None = None, shared_gate: torch.Tensor | None = None) -> torch.Tensor:
+                         out: torch.Tensor, shared: torch.Tensor | None = None, shared_gate: torch.Tensor | None = None,
+                         gated: bool = False) -> torch.Tensor:
     """out[t] = sum over the token's ``top`` pairs of weight[t, k] * (Wd[e] relu(Wu[e] x[t])^2, or x[t] itself for a pair
     without a slot) + sigmoid(shared_gate[t]) * shared[t]. w_up [E, F, K], w_down [E, N, F] (both None: every expert stands
-    for the input); ``routed`` from ``moe_route_chosen``; shared float32 [T, N] or None; shared_gate a float32 view [T, >= 1]."""
+    for the input); ``routed`` from ``moe_route_chosen``; shared float32 [T, N] or None; shared_gate a float32 view [T, >= 1].
+    ``gated``: an expert is Wd[e] (silu(Wg[e] x) * (Wu[e] x)) and w_up is [E, 2F, K], an expert's gate rows, then its up rows."""
     slot_pair, pair_slot, tiles, n_tiles, tile_rows = routed
     _gpu(x, w_up, w_down, out, weight, shared, shared_gate)
     T, K = x.shape
@@ -1801,20 +1839,125 @@ def moe_experts_weighted(x: torch.Tensor, routed, weight: torch.Tensor, w_up: to
     part = torch.empty((max(P, 1), N), dtype=torch.float32, device=x.device)
     if w_up is not None and most > 0:
         E, F, K2 = w_up.shape
+        if gated:
+            _need(F % 2 == 0, "moe_experts_weighted: gate rows and up rows come in equal numbers")
+            F //= 2
         _need(K2 == K and tuple(w_down.shape) == (E, N, F) and w_up.is_contiguous() and w_down.is_contiguous()
               and x.dtype == w_up.dtype == w_down.dtype, "moe_experts_weighted: w_up [E, F, K], w_down [E, N, F], one type")
         act = torch.empty((P, F), dtype=x.dtype, device=x.device)
         if x.dtype == torch.bfloat16 and lib.tm_moe_mfma_takes(_p(x), c_int(ldx), _p(w_up), _p(w_down), _p(act), c_int(K), c_int(F)):
-            _check(lib.tm_moe_up_act_mfma(_p(x), c_int(ldx), _p(slot_pair), c_int(top), _p(w_up), _p(act), _p(tiles), _p(n_tiles),
-                                          c_int(most), c_int(tile_rows), c_int(K), c_int(F), _stream()), "moe_up_act_mfma")
+            first = lib.tm_moe_gate_up_mfma if gated else lib.tm_moe_up_act_mfma
+            _check(first(_p(x), c_int(ldx), _p(slot_pair), c_int(top), _p(w_up), _p(act), _p(tiles), _p(n_tiles),
+                         c_int(most), c_int(tile_rows), c_int(K), c_int(F), _stream()), "moe_up_act_mfma")
             _check(lib.tm_moe_down_mfma(_p(act), _p(w_down), _p(part), _p(tiles), _p(n_tiles), c_int(most), c_int(tile_rows), c_int(F),
                                         c_int(N), _stream()), "moe_down_mfma")
         else:
             _need(tile_rows == MOE_TILE_ROWS, "moe_experts_weighted: these products take tiles of 32 rows")
-            _check(lib.tm_moe_up_act(_p(x), c_int(ldx), _p(slot_pair), c_int(top), _p(w_up), _p(act), _p(tiles), _p(n_tiles), c_int(most),
-                                     c_int(K), c_int(F), dt, _stream()), "moe_up_act")
+            first = lib.tm_moe_gate_up if gated else lib.tm_moe_up_act
+            _check(first(_p(x), c_int(ldx), _p(slot_pair), c_int(top), _p(w_up), _p(act), _p(tiles), _p(n_tiles), c_int(most),
+                         c_int(K), c_int(F), dt, _stream()), "moe_up_act")
             _check(lib.tm_moe_down(_p(act), _p(w_down), _p(part), _p(tiles), _p(n_tiles), c_int(most), c_int(F), c_int(N), dt, _stream()),
                    "moe_down")
     _check(lib.tm_moe_combine_weighted(_p(part), _p(pair_slot), _p(weight), _p(x), c_int(ldx), _p(shared), _p(shared_gate), c_int(ldg),
                                        _p(out), c_int(T), c_int(top), c_int(N), dt, _stream()), "moe_combine_weighted")
+    return out
+
+
+# -------------------------------------------------------------------------------------------- the gated delta rule
+
+DELTA_MAX_KEY_DIM = 256
+DELTA_MAX_CHANNELS = 16384          # convolved channels of a token (q | k | v): what a block keeps in LDS
+
+
+def delta_row_width(H: int, G: int, D: int, Dv: int) -> int:
+    """Floats of a prepared row [q | k | v | beta | g | k.q], rounded up to whole 16-byte pieces."""
+    return -(-(2 * G * D + H * Dv + 2 * H + G) // 4) * 4
+
+
+def delta_prepare(proj: torch.Tensor, conv_w: torch.Tensor, conv_state: torch.Tensor | None, ba: torch.Tensor, a_log: torch.Tensor,
+                  dt_bias: torch.Tensor, cu_q_lens: torch.Tensor, state_slots: torch.Tensor, seq_of_token: torch.Tensor, num_seqs: int,
+                  out: torch.Tensor, H: int, G: int, D: int, Dv: int, unit_eps: float = 1e-6) -> torch.Tensor:
+    """The rows the delta-rule recurrence reads, from the projections of a step. proj [T, >= C] (C = 2 G D + H Dv: the q, k and v
+    channels first) in the model's type; conv_w [C, taps] and conv_state [slots, taps - 1, C] of the same type (the rows before a
+    request's first row of the step come from its state; the state itself is advanced by ``delta_conv_state``); ba float32
+    [T, >= 2H] = [b | a]; a_log, dt_bias float32 [H]. Per token: y = silu(conv(.)), q = y_q / sqrt(sum y_q^2 + eps) / sqrt(D),
+    k = y_k / sqrt(sum y_k^2 + eps), beta = sigmoid(b), g = exp(-exp(a_log) softplus(a + dt_bias)); out float32
+    [T, delta_row_width] = [q | k | v | beta | g | k.q]."""
+    _gpu(proj, conv_w, conv_state, ba, a_log, dt_bias, cu_q_lens, state_slots, seq_of_token, out)
+    T = proj.shape[0]
+    C = 2 * G * D + H * Dv
+    taps = conv_w.shape[1]
+    _need(proj.dim() == 2 and proj.stride(1) == 1 and proj.shape[1] >= C, f"delta_prepare: proj is [T, >= {C}]")
+    _need(H % G == 0 and 0 < D <= DELTA_MAX_KEY_DIM and C <= DELTA_MAX_CHANNELS, "delta_prepare: sizes the kernels do not take")
+    _need(tuple(conv_w.shape) == (C, taps) and conv_w.is_contiguous() and conv_w.dtype == proj.dtype and 1 <= taps <= 16,
+          f"delta_prepare: conv_w is [{C}, taps] of proj's type, taps up to 16")
+    if taps > 1:
+        _need(conv_state is not None and conv_state.dim() == 3 and tuple(conv_state.shape[1:]) == (taps - 1, C)
+              and conv_state.is_contiguous() and conv_state.dtype == proj.dtype, f"delta_prepare: conv_state is [slots, {taps - 1}, {C}] of proj's type")
+    _need(ba.dtype == torch.float32 and ba.dim() == 2 and ba.shape[0] == T and ba.shape[1] >= 2 * H and ba.stride(1) == 1,
+          f"delta_prepare: ba is float32 [T, >= {2 * H}]")
+    for name, v in (("a_log", a_log), ("dt_bias", dt_bias)):
+        _need(v.dtype == torch.float32 and tuple(v.shape) == (H,) and v.is_contiguous(), f"delta_prepare: {name} is float32 [{H}]")
+    ldo = out.shape[1] if out.dim() == 2 else 0
+    _need(out.dtype == torch.float32 and out.dim() == 2 and out.shape[0] == T and out.is_contiguous() and ldo >= C + 2 * H + G,
+          "delta_prepare: out is contiguous float32 [T, >= C + 2H + G]")
+    _ints(cu_q_lens, num_seqs + 1, "cu_q_lens")
+    _ints(state_slots, num_seqs, "state_slots")
+    _ints(seq_of_token, T, "seq_of_token")
+    ld = proj.stride(0) if T > 1 else max(proj.stride(0), proj.shape[1])
+    ldba = ba.stride(0) if T > 1 else max(ba.stride(0), ba.shape[1])
+    _check(library().tm_delta_prepare(_p(proj), c_int(ld), _p(conv_w), _p(conv_state), _p(ba), c_int(ldba), _p(a_log), _p(dt_bias),
+                                      _p(cu_q_lens), _p(state_slots), _p(seq_of_token), _p(out), c_int(ldo), c_int(T), c_int(H), c_int(G),
+                                      c_int(D), c_int(Dv), c_int(taps), c_float(unit_eps), c_int(code(proj.dtype)), _stream()),
+           "delta_prepare")
+    return out
+
+
+def delta_conv_state(proj: torch.Tensor, C: int, conv_state: torch.Tensor, cu_q_lens: torch.Tensor, state_slots: torch.Tensor,
+                     num_seqs: int) -> None:
+    """Every request's convolution state [taps - 1, C] becomes the last taps - 1 rows it has seen (the first C columns of proj)."""
+    _gpu(proj, conv_state, cu_q_lens, state_slots)
+    T = proj.shape[0]
+    _need(conv_state.dim() == 3 and conv_state.shape[2] == C and conv_state.is_contiguous() and conv_state.dtype == proj.dtype,
+          f"delta_conv_state: the state is [slots, taps - 1, {C}] of proj's type")
+    _need(proj.dim() == 2 and proj.stride(1) == 1 and proj.shape[1] >= C, f"delta_conv_state: proj is [T, >= {C}]")
+    _ints(cu_q_lens, num_seqs + 1, "cu_q_lens")
+    _ints(state_slots, num_seqs, "state_slots")
+    ld = proj.stride(0) if T > 1 else max(proj.stride(0), proj.shape[1])
+    _check(library().tm_delta_conv_state(_p(proj), c_int(ld), _p(conv_state), _p(cu_q_lens), _p(state_slots), c_int(num_seqs), c_int(C),
+                                         c_int(conv_state.shape[1] + 1), c_int(code(proj.dtype)), _stream()), "delta_conv_state")
+
+
+def delta_scan(rows: torch.Tensor, o: torch.Tensor, state: torch.Tensor, cu_q_lens: torch.Tensor, state_slots: torch.Tensor,
+               num_seqs: int, H: int, G: int, D: int, Dv: int) -> torch.Tensor:
+    """The recurrence over the rows of ``delta_prepare``, request by request in the order of the step's rows:
+    S <- g S; u = beta (v - S^T k); S <- S + k u^T; o = S^T q. state float32 [slots, H, D, Dv] (row state_slots[s] is read and
+    written); o float32 [T, H * Dv]."""
+    _gpu(rows, o, state, cu_q_lens, state_slots)
+    T = rows.shape[0]
+    _need(rows.dtype == torch.float32 and rows.dim() == 2 and rows.is_contiguous() and rows.shape[1] >= 2 * G * D + H * Dv + 2 * H + G,
+          "delta_scan: rows are those of delta_prepare")
+    _need(o.dtype == torch.float32 and o.is_contiguous() and tuple(o.shape) == (T, H * Dv), f"delta_scan: o is float32 [{T}, {H * Dv}]")
+    _need(state.dtype == torch.float32 and state.is_contiguous() and tuple(state.shape[1:]) == (H, D, Dv),
+          f"delta_scan: state is float32 [slots, {H}, {D}, {Dv}]")
+    _need(H % G == 0 and 0 < D <= DELTA_MAX_KEY_DIM, "delta_scan: sizes the kernel does not take")
+    _ints(cu_q_lens, num_seqs + 1, "cu_q_lens")
+    _ints(state_slots, num_seqs, "state_slots")
+    _check(library().tm_delta_scan(_p(rows), c_int(rows.shape[1]), _p(o), _p(state), _p(cu_q_lens), _p(state_slots), c_int(num_seqs),
+                                   c_int(H), c_int(G), c_int(D), c_int(Dv), _stream()), "delta_scan")
+    return o
+
+
+def pair_norm_mean(a: torch.Tensor, b: torch.Tensor, wa: torch.Tensor, wb: torch.Tensor, out: torch.Tensor, eps: float) -> torch.Tensor:
+    """out = (a / rms(a) * wa + b / rms(b) * wb) / 2 row by row, statistics and sums in 32-bit; a, b, out [T, W] of one type,
+    wa, wb float32 [W]."""
+    _gpu(a, b, wa, wb, out)
+    T, W = a.shape
+    _need(a.is_contiguous() and b.is_contiguous() and out.is_contiguous() and a.shape == b.shape == out.shape
+          and a.dtype == b.dtype == out.dtype, "pair_norm_mean: a, b and out are contiguous, of one shape and type")
+    for w in (wa, wb):
+        _need(w.dtype == torch.float32 and tuple(w.shape) == (W,) and w.is_contiguous(), f"pair_norm_mean: the weights are float32 [{W}]")
+    _need(eps > 0, "pair_norm_mean: eps must be positive")
+    _check(library().tm_pair_norm_mean(_p(a), _p(b), _p(wa), _p(wb), _p(out), c_int(T), c_int(W), c_float(eps), c_int(code(a.dtype)),
+                                       _stream()), "pair_norm_mean")
     return out

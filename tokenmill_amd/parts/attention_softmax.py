@@ -3,7 +3,8 @@
   * grouped key/value heads and values of another size than keys;
   * biases on q, k and v;
   * an RMS norm of q and of k over the WHOLE projection (all heads of a token at once, one weight per channel of the
-    projection), before the rotation;
+    projection), before the rotation; or instead an RMS norm of every head of q and of k by itself, with one weight per
+    channel of a head that the heads share;
   * a rotation of the first channels of each head, pairs a half apart or neighbouring, with whatever frequencies the
     ``RotaryEmbedding`` was built with;
   * scores capped smoothly: s <- cap * tanh(s / cap);
@@ -34,11 +35,15 @@ class SoftmaxAttention(Mixer):
     def __init__(self, hidden: int, num_heads: int, num_kv_heads: int, head_dim: int, v_head_dim: int, scale: float,
                  rotary: RotaryEmbedding | None = None, whole_norm_eps: float | None = None, qkv_bias: bool = False,
                  softcap: float | None = None, head_gate: bool = False, window: int | None = None, own_kv: bool = True,
+                 head_norm_eps: float | None = None,
                  names: tuple[str, str, str, str] = ("q", "k", "v", "o"),
                  extra_names: tuple[str, str, str] = ("q.norm", "k.norm", "g"),
                  suffixes: tuple[str, str] = ("", ".b")):
-        """``whole_norm_eps``: None for no norm of q and k. ``softcap``: None or 0 for none. ``extra_names``: the
-        checkpoint's names of the two norm weights and of the gate's matrix, under the mixer's prefix."""
+        """``whole_norm_eps``: None for no norm of q and k over the whole projection; ``head_norm_eps``: None for no norm head
+        by head (one of the two at most). ``softcap``: None or 0 for none. ``extra_names``: the checkpoint's names of the two
+        norm weights and of the gate's matrix, under the mixer's prefix."""
+        if whole_norm_eps is not None and head_norm_eps is not None:
+            raise ValueError("q and k are normed over the whole projection or head by head, not both")
         if num_heads % num_kv_heads:
             raise ValueError(f"{num_heads} query heads do not divide into {num_kv_heads} kv heads")
         if head_dim % 4 or not 0 < head_dim <= MAX_HEAD_DIM or not 0 < v_head_dim <= MAX_HEAD_DIM:
@@ -52,6 +57,8 @@ class SoftmaxAttention(Mixer):
         self.hidden, self.num_heads, self.num_kv_heads = hidden, num_heads, num_kv_heads
         self.head_dim, self.v_head_dim = head_dim, v_head_dim
         self.scale, self.rotary, self.whole_norm_eps = float(scale), rotary, whole_norm_eps
+        self.head_norm_eps = head_norm_eps
+        self.norm_eps = whole_norm_eps if whole_norm_eps is not None else head_norm_eps     # None: q and k are not normed
         self.softcap, self.window, self.own_kv = float(softcap or 0.0), window, own_kv
         self.q_size, self.k_size, self.v_size = num_heads * head_dim, num_kv_heads * head_dim, num_kv_heads * v_head_dim
         sizes, stacked = [self.q_size], [names[0]]
@@ -81,17 +88,18 @@ class SoftmaxAttention(Mixer):
         for lin in self._linears():
             specs.update(lin.tensor_specs(prefix))
         qn, kn, _ = self.extra_names
-        if self.whole_norm_eps is not None:
-            specs[prefix + qn] = TensorSpec((self.q_size,), init="ones")
+        if self.norm_eps is not None:
+            per_head = self.head_norm_eps is not None
+            specs[prefix + qn] = TensorSpec((self.head_dim if per_head else self.q_size,), init="ones")
             if self.own_kv:
-                specs[prefix + kn] = TensorSpec((self.k_size,), init="ones")
+                specs[prefix + kn] = TensorSpec((self.head_dim if per_head else self.k_size,), init="ones")
         return specs
 
     def load(self, tensors, prefix: str) -> None:
         for lin in self._linears():
             lin.load(tensors, prefix)
         qn, kn, _ = self.extra_names
-        if self.whole_norm_eps is not None:         # the vectors that meet 32-bit statistics are kept in 32-bit
+        if self.norm_eps is not None:               # the vectors that meet 32-bit statistics are kept in 32-bit
             self.q_norm = tensors[prefix + qn].float().contiguous()
             self.k_norm = tensors[prefix + kn].float().contiguous() if self.own_kv else None
         if self.rotary is not None:
@@ -148,10 +156,11 @@ class SoftmaxAttention(Mixer):
             elif self.gate is not None:
                 gate = self.gate.forward(x, out_dtype=torch.float32)
             q = torch.empty((T, self.q_size), dtype=x.dtype, device=x.device)
-            ops.whole_norm_rope_store(proj, q, H, G, D, Dv, self.q_norm, self.k_norm, self.whole_norm_eps or 1.0,
+            ops.whole_norm_rope_store(proj, q, H, G, D, Dv, self.q_norm, self.k_norm, self.norm_eps or 1.0,
                                       rot.cos if rot is not None else None, rot.sin if rot is not None else None,
                                       bool(rot is not None and rot.interleaved), step.positions, group.slot_mapping,
-                                      cache.k if self.own_kv else None, cache.v if self.own_kv else None, has_kv=self.own_kv)
+                                      cache.k if self.own_kv else None, cache.v if self.own_kv else None, has_kv=self.own_kv,
+                                      per_head=self.head_norm_eps is not None)
         if D == Dv:
             # keys and values of one size: the kernel library's own attention operation, which is handed q and chooses the
             # kernels of a step (prompt portions and single tokens on the matrix unit where it takes the sizes), then

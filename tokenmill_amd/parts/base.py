@@ -62,9 +62,10 @@ class StateSpec:
 @dataclass(frozen=True)
 class LayerCacheSpec:
     """What a layer needs when it is more than one thing: pages for its mixer's keys and a slot of state beside them
-    (a short convolution in front of an attention). Either may be None."""
+    (a short convolution in front of an attention; two mixers side by side). Either may be None. ``state`` may be a tuple of
+    specs: the layer then gets a tuple of tensors, one per spec."""
     kv: KVCacheSpec | None = None
-    state: StateSpec | None = None
+    state: StateSpec | tuple | None = None
 
 
 @dataclass
@@ -74,12 +75,12 @@ class KVCacheView:
     v: torch.Tensor | None       # [pages, kv_heads, value size, page_size]; None for a group without a value pool
     group: int                   # index into StepContext.groups
     write: bool = True           # False: this layer reads a cache that another layer writes
-    state: torch.Tensor | None = None    # [slots, *shape] of a layer that keeps state beside its pages
+    state: torch.Tensor | tuple | None = None    # [slots, *shape] of a layer that keeps state beside its pages (a tuple: several)
 
 
 @dataclass
 class StateView:
-    state: torch.Tensor          # [slots, *shape]; row StepContext.state_slots[s] belongs to request s
+    state: torch.Tensor | tuple  # [slots, *shape]; row StepContext.state_slots[s] belongs to request s (a tuple: several states)
 
 
 # ------------------------------------------------------------------------------------------------

@@ -25,11 +25,13 @@ class LearnedPositions(Part):
 
 
 class TokenEmbedding(Part):
-    """x = E[ids], no scaling; rows are widened into the 32-bit residual stream. With ``places`` (a
-    ``LearnedPositions``) the row of the token's position is added, in 32-bit."""
+    """x = E[ids] * scale (``scale`` 1 unless the model says otherwise); rows are widened into the 32-bit residual stream.
+    With ``places`` (a ``LearnedPositions``) the row of the token's position is added, in 32-bit."""
 
-    def __init__(self, vocab: int, hidden: int, name: str = "weight", places: LearnedPositions | None = None):
-        self.vocab, self.hidden, self.name, self.places = vocab, hidden, name, places
+    def __init__(self, vocab: int, hidden: int, name: str = "weight", places: LearnedPositions | None = None, scale: float = 1.0):
+        if places is not None and scale != 1.0:
+            raise ValueError("an embedding with position rows has no scale")
+        self.vocab, self.hidden, self.name, self.places, self.scale = vocab, hidden, name, places, float(scale)
         self.weight: torch.Tensor | None = None
 
     @property
@@ -49,8 +51,8 @@ class TokenEmbedding(Part):
             self.places.load(tensors, prefix)
 
     def emit(self, program) -> int | None:
-        if self.places is not None:
-            return None                         # the library's operation gathers token rows only
+        if self.places is not None or self.scale != 1.0:
+            return None                         # the library's operation gathers token rows only, as they are
         return program.embedding(self, self.weight)
 
     def cost(self, label, step, rows):
@@ -61,7 +63,7 @@ class TokenEmbedding(Part):
         with profiling.label("embed", lambda: self.cost("embed", None, token_ids.numel())):
             if self.places is not None:
                 return ops.embed_gather_pos(self.weight, self.places.weight, token_ids, positions, out)
-            return ops.embed_gather(self.weight, token_ids, out)
+            return ops.embed_gather(self.weight, token_ids, out, self.scale)
 
 
 class OutputHead(Part):

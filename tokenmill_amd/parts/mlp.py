@@ -118,3 +118,44 @@ class DenseFeedForward(FeedForward):
                 ops.gelu_tanh(a, a)
         with profiling.label("down", lambda: self.down.cost(x.shape[0])):
             return self.down.forward(a)
+
+
+class GatedFeedForward(FeedForward):
+    """down(act(gate(x)) * up(x)) without biases, gate and up stacked into one product. ``activation``: "gelu_tanh", the
+    tanh form of GELU, or "silu"; it is computed in 32-bit on the gate's rounded result and the product with up is rounded
+    once. (``SwiGLU`` is the "silu" case as one operation of the kernel library's step program, for models whose blocks
+    describe themselves to it.)"""
+
+    ACTIVATIONS = ("gelu_tanh", "silu")
+
+    def __init__(self, hidden: int, intermediate: int, activation: str = "gelu_tanh", names: tuple[str, str, str] = ("gate", "up", "down"),
+                 suffixes: tuple[str, str] = ("", ".b")):
+        if activation not in self.ACTIVATIONS:
+            raise ValueError(f"activation '{activation}' is not one of {sorted(self.ACTIVATIONS)}")
+        self.hidden, self.intermediate, self.activation = hidden, intermediate, activation
+        self.gate_up = Linear(hidden, [intermediate, intermediate], list(names[:2]), bias=False, suffixes=suffixes)
+        self.down = Linear(intermediate, hidden, names[2], bias=False, suffixes=suffixes)
+
+    def tensor_specs(self, prefix: str):
+        return {**self.gate_up.tensor_specs(prefix), **self.down.tensor_specs(prefix)}
+
+    def load(self, tensors, prefix: str) -> None:
+        self.gate_up.load(tensors, prefix)
+        self.down.load(tensors, prefix)
+
+    def prepare(self, pack_weights: bool) -> None:
+        self.gate_up.prepare(pack_weights)
+        self.down.prepare(pack_weights)
+
+    def cost(self, label: str, step: StepContext | None, rows: int) -> tuple[int, int]:
+        return self.gate_up.cost(rows) if label == "gate_up" else self.down.cost(rows)
+
+    def forward(self, x, step: StepContext | None = None, residual: torch.Tensor | None = None):
+        from tokenmill_amd import profiling
+        x = as_tensor(x)
+        with profiling.label("gate_up", lambda: self.gate_up.cost(x.shape[0])):
+            gu = self.gate_up.forward(x)
+            a = torch.empty((x.shape[0], self.intermediate), dtype=x.dtype, device=x.device)
+            (ops.gelu_mul if self.activation == "gelu_tanh" else ops.silu_mul)(gu, a)
+        with profiling.label("down", lambda: self.down.cost(x.shape[0])):
+            return self.down.forward(a)

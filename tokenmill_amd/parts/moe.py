@@ -81,25 +81,42 @@ class TableRoutedExperts(FeedForward):
 
 class RoutedExperts(FeedForward):
     """Experts chosen by a learned router, each W_down act(W_up x) without biases (``activation``: "relu2", the square of
-    relu), plus what a model may add around them:
+    relu; or "swiglu": W_down (silu(W_gate x) * (W_up x)), with ``names`` then (gate, up, down)), plus what a model may add
+    around them:
 
       z = W_router x (32-bit);  s = softmax(z) over all router outputs;  the ``top`` largest of s + correction are chosen
       (``correction``: a stored vector that shifts the choice only);  weight = s of the chosen / (their sum + 1e-20)
       the last ``identity`` router outputs are experts without matrices: their output is x itself
       y = sum of weight * expert(x)  +  sigmoid(w_sg . x) * shared(x)      (``shared_ff``: the width of an expert of the same
       form that every token uses; None for none; ``shared_gate`` False: the shared result is added as it is)
+      ``scoring`` "chosen_logits": the ``top`` largest z themselves are chosen and the weights are the softmax over the chosen z
+      only (no correction); ``router_bias``: z = W_router x + b, the bias added in 32-bit
 
     The router's rows and the shared gate's row are one 32-bit product. The step's (token, expert) pairs are sorted by expert
     on the device and every expert multiplies its own rows in tiles; nothing about the routing crosses to the host."""
 
-    ACTIVATIONS = ("relu2",)
+    ACTIVATIONS = ("relu2", "swiglu")
+    SCORINGS = ("softmax", "chosen_logits")
 
     def __init__(self, hidden: int, intermediate: int, experts: int, top: int, identity: int = 0, correction: bool = True,
                  shared_ff: int | None = None, shared_gate: bool = True, activation: str = "relu2",
-                 names: tuple[str, str] = ("up", "down"), expert_prefix: str = "e{e}.", router_name: str = "router",
-                 correction_name: str = "correction", shared_prefix: str = "shared.", shared_gate_name: str = "shared.sg"):
+                 names: tuple[str, ...] | None = None, expert_prefix: str = "e{e}.", router_name: str = "router",
+                 correction_name: str = "correction", shared_prefix: str = "shared.", shared_gate_name: str = "shared.sg",
+                 scoring: str = "softmax", router_bias: bool = False):
         if activation not in self.ACTIVATIONS:
             raise ValueError(f"activation '{activation}' is not one of {list(self.ACTIVATIONS)}")
+        if scoring not in self.SCORINGS:
+            raise ValueError(f"scoring '{scoring}' is not one of {list(self.SCORINGS)}")
+        if scoring == "chosen_logits" and correction:
+            raise ValueError("a correction shifts a choice among softmax scores; the chosen-logits scoring has none")
+        self.gated = activation == "swiglu"
+        if names is None:
+            names = ("gate", "up", "down") if self.gated else ("up", "down")
+        if len(names) != (3 if self.gated else 2):
+            raise ValueError("an expert's tensors are (up, down), or (gate, up, down) with a gate")
+        if self.gated and shared_ff:
+            raise ValueError("a shared expert with a gate of its own is not arranged for")
+        self.scoring = scoring
         if experts < 0 or identity < 0 or not 0 < top <= experts + identity <= ops.MOE_MAX_EXPERTS:
             raise ValueError(f"{top} of {experts} + {identity} experts: a token uses at least one and at most all, of up to {ops.MOE_MAX_EXPERTS}")
         self.hidden, self.intermediate, self.experts, self.identity, self.top = hidden, intermediate, experts, identity, top
@@ -111,10 +128,12 @@ class RoutedExperts(FeedForward):
         if self.has_shared_gate:
             rows.append(1)
             stacked.append(shared_gate_name)
-        self.router = Linear(hidden, rows, stacked, bias=False, suffixes=("", ".b"))
+        if router_bias and self.has_shared_gate:
+            raise ValueError("a router with a bias beside a shared gate is not arranged for")
+        self.router = Linear(hidden, rows, stacked, bias=router_bias, suffixes=("", ".b"), wide_bias=True)
         self.shared_up = Linear(hidden, shared_ff, shared_prefix + names[0], bias=False, suffixes=("", ".b"), activation="relu2") if shared_ff else None
         self.shared_down = Linear(shared_ff, hidden, shared_prefix + names[1], bias=False, suffixes=("", ".b")) if shared_ff else None
-        self.up: torch.Tensor | None = None             # [E, F, hidden]
+        self.up: torch.Tensor | None = None             # [E, F, hidden]; with a gate [E, 2 F, hidden]: an expert's gate rows, then its up rows
         self.down: torch.Tensor | None = None           # [E, hidden, F]
         self.correction: torch.Tensor | None = None     # float32 [experts + identity]
 
@@ -132,14 +151,19 @@ class RoutedExperts(FeedForward):
         if self.has_correction:
             specs[prefix + self.correction_name] = TensorSpec((self.outputs,))
         for e in range(self.experts):
-            specs[self._name(prefix, e, 0)] = TensorSpec((F, W))
-            specs[self._name(prefix, e, 1)] = TensorSpec((W, F))
+            for which in range(len(self.names) - 1):
+                specs[self._name(prefix, e, which)] = TensorSpec((F, W))
+            specs[self._name(prefix, e, len(self.names) - 1)] = TensorSpec((W, F))
         return specs
 
     def load(self, tensors, prefix: str) -> None:
         for lin in self._linears():
             lin.load(tensors, prefix)
-        if self.experts:
+        if self.experts and self.gated:
+            self.up = torch.stack([torch.cat([tensors[self._name(prefix, e, 0)], tensors[self._name(prefix, e, 1)]])
+                                   for e in range(self.experts)]).contiguous()
+            self.down = torch.stack([tensors[self._name(prefix, e, 2)] for e in range(self.experts)]).contiguous()
+        elif self.experts:
             self.up = torch.stack([tensors[self._name(prefix, e, 0)] for e in range(self.experts)]).contiguous()
             self.down = torch.stack([tensors[self._name(prefix, e, 1)] for e in range(self.experts)]).contiguous()
         if self.has_correction:
@@ -161,8 +185,9 @@ class RoutedExperts(FeedForward):
             m2, f2 = self.shared_down.cost(rows, out_bytes=4)
             return m1 + m2, f1 + f2
         used = min(self.experts, rows * self.top)
-        moved = used * 2 * self.intermediate * self.hidden * e + rows * self.hidden * 2 * e + rows * self.top * self.intermediate * 2 * e
-        return moved, 4 * rows * self.top * self.intermediate * self.hidden
+        mats = 3 if self.gated else 2
+        moved = used * mats * self.intermediate * self.hidden * e + rows * self.hidden * 2 * e + rows * self.top * self.intermediate * 2 * e
+        return moved, 2 * mats * rows * self.top * self.intermediate * self.hidden
 
     def forward(self, x, step: StepContext, residual: torch.Tensor | None = None):
         x = as_tensor(x)
@@ -170,7 +195,7 @@ class RoutedExperts(FeedForward):
         out = torch.empty((T, self.hidden), dtype=x.dtype, device=x.device)
         with profiling.label("router", lambda: self.cost("router", step, T)):
             z = self.router.forward(x, out_dtype=torch.float32)
-            chosen, weight = ops.moe_router(z, self.outputs, self.top, self.correction)
+            chosen, weight = ops.moe_router(z, self.outputs, self.top, self.correction, over_chosen=self.scoring == "chosen_logits")
         shared = None
         if self.shared_up is not None:
             with profiling.label("shared", lambda: self.cost("shared", step, T)):
@@ -181,4 +206,4 @@ class RoutedExperts(FeedForward):
             rows = ops.moe_tile_rows(T * self.top, max(self.experts, 1), x.dtype) if mfma else ops.MOE_TILE_ROWS
             routed = ops.moe_route_chosen(chosen, self.outputs, self.experts, rows)
             gate = z[:, self.outputs:self.outputs + 1] if self.has_shared_gate else None
-            return ops.moe_experts_weighted(x, routed, weight, self.up, self.down, self.top, out, shared, gate)
+            return ops.moe_experts_weighted(x, routed, weight, self.up, self.down, self.top, out, shared, gate, gated=self.gated)

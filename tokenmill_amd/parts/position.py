@@ -26,13 +26,15 @@ class RotaryEmbedding(PositionEncoding):
         are blended linearly over the pair index; cos and sin are multiplied by 0.1 ln(factor) + 1. With j(t) =
         rotary_dim * ln(original / (2 pi t)) / (2 ln theta): lo = max(floor(j(fast)), 0), hi = min(ceil(j(slow)),
         rotary_dim - 1), ramp_i = clamp((i - lo) / max(hi - lo, 0.001), 0, 1), f_i <- f_i / factor * ramp_i + f_i (1 - ramp_i).
-        ``exact``: the frequencies are computed in 64-bit and rounded once to 32-bit (always so with ``scaling``)."""
+        A ``scaling`` that holds a ``factor`` alone is linear: every frequency is divided by the factor, cos and sin stay as
+        they are. ``exact``: the frequencies are computed in 64-bit and rounded once to 32-bit (always so with ``scaling``)."""
         self.head_dim = head_dim
         self.interleaved = interleaved
         self.scaling = dict(scaling) if scaling else None
         self.exact = exact or self.scaling is not None
+        self.linear = self.scaling is not None and set(self.scaling) == {"factor"}
         if self.scaling is not None:
-            for key in ("factor", "original", "fast", "slow"):
+            for key in ("factor",) if self.linear else ("factor", "original", "fast", "slow"):
                 if key not in self.scaling:
                     raise ValueError(f"rotary scaling has no '{key}'")
             if not float(self.scaling["factor"]) > 0:
@@ -55,6 +57,8 @@ class RotaryEmbedding(PositionEncoding):
         sc = self.scaling
         if sc is None:
             return f.float(), 1.0
+        if self.linear:
+            return (f / float(sc["factor"])).float(), 1.0
         factor, original = float(sc["factor"]), float(sc["original"])
 
         def pair_of(turns: float) -> float:
