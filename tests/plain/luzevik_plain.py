@@ -2,8 +2,8 @@
 
 It shares no code with the engine: it reads a config dictionary and a dictionary of tensors and computes with ordinary
 tensor expressions. ``dtype`` says what the engine's storage type is; the places where the engine rounds to it are the
-places where ``rnd`` is applied here (inputs and results of matrix products, cached rows, the short convolution), and
-everything else is 32-bit.
+places where ``rnd`` is applied here (inputs of matrix products and those of their results that the engine stores, cached
+rows, rotated queries, each sublayer's result), and everything else is 32-bit.
 
 Notation: x is the 32-bit residual stream [T, W]; a layer is
     x += unit(mixer(x)) * w1;   x += unit(ff(x)) * w2          (the second only with a feed-forward)
@@ -55,9 +55,9 @@ def frequencies(rot: dict):
     return f.float()
 
 
-def rotate_half(v, positions, rot: dict):
+def rotate_half(v, positions, rot: dict | None):
     """v [T, heads, D]: of every head's first rot.dims channels, channel i and channel i + dims/2 turn as a pair."""
-    dims = int(rot["dims"])
+    dims = int(rot["dims"]) if rot else 0
     if dims == 0:
         return v
     a = positions.float()[:, None] * frequencies(rot)[None, :]
@@ -90,7 +90,7 @@ def latent_rows(h, m, t, pre, eps, positions, dtype):
     R, Dr = int(m["kv_rank"]), int(m["rot_dim"])
     low = linear(h, t[pre + "dkv"], dtype=dtype)
     c = rnd(rms(low[:, :R], t[pre + "dkv.norm"], eps), dtype)
-    kr = rotate_half(low[:, None, R:R + Dr], positions, m["rot"])[:, 0]
+    kr = rotate_half(low[:, None, R:R + Dr], positions, m.get("rot"))[:, 0]
     return c, rnd(kr, dtype)
 
 
@@ -100,13 +100,13 @@ def latent_attention(h, m, t, pre, eps, positions, rows, dtype):
     H, D, Dr, Dv = int(m["heads"]), int(m["dim"]), int(m["rot_dim"]), int(m["vdim"])
     c, kr = rows
     cq = rnd(rms(linear(h, t[pre + "dq"], dtype=dtype), t[pre + "dq.norm"], eps), dtype)
-    q = linear(cq, t[pre + "uq"], dtype=dtype).view(T, H, D + Dr)
-    qn, qr = q[..., :D], rotate_half(q[..., D:], positions, m["rot"])
+    q = rnd(linear(cq, t[pre + "uq"], dtype=dtype), dtype).view(T, H, D + Dr)
+    qn, qr = q[..., :D], rnd(rotate_half(q[..., D:], positions, m.get("rot")), dtype)
     kn = (c @ t[pre + "uk"].float().T).view(T, H, D)
     v = (c @ t[pre + "uv"].float().T).view(T, H, Dv)
     k = torch.cat([kn, kr[:, None, :].expand(T, H, Dr)], dim=-1)
     o = softmax_attention(torch.cat([qn, qr], dim=-1), k, v, float(m["scale"]), sink=t[pre + "sink"])
-    return linear(o.reshape(T, H * Dv), t[pre + "o"], dtype=dtype)
+    return rnd(linear(o.reshape(T, H * Dv), t[pre + "o"], dtype=dtype), dtype)
 
 
 def grouped_attention(h, m, t, pre, eps, positions, dtype):
@@ -116,19 +116,21 @@ def grouped_attention(h, m, t, pre, eps, positions, dtype):
     q = linear(h, t[pre + "q"], t[pre + "q.b"], dtype).view(T, H, D)
     k = linear(h, t[pre + "k"], t[pre + "k.b"], dtype).view(T, G, D)
     v = rnd(linear(h, t[pre + "v"], t[pre + "v.b"], dtype), dtype).view(T, G, Dv)
-    q = rnd(rotate_half(rms(q, t[pre + "q.norm"], eps), positions, m["rot"]), dtype)
-    k = rnd(rotate_half(rms(k, t[pre + "k.norm"], eps), positions, m["rot"]), dtype)
+    q = rnd(rotate_half(rms(q, t[pre + "q.norm"], eps), positions, m.get("rot")), dtype)
+    k = rnd(rotate_half(rms(k, t[pre + "k.norm"], eps), positions, m.get("rot")), dtype)
     k, v = k.repeat_interleave(H // G, dim=1), v.repeat_interleave(H // G, dim=1)
     o = softmax_attention(q, k, v, float(m["scale"]))
-    return linear(o.reshape(T, H * Dv), t[pre + "o"], dtype=dtype)
+    return rnd(linear(o.reshape(T, H * Dv), t[pre + "o"], dtype=dtype), dtype)
 
 
-def conv_silu(u, w, dtype):
-    """u [T, C], w [C, taps]: y_t = silu(sum_j w[:, j] u_(t - taps + 1 + j)), zeros before the first token."""
+def conv_silu(u, w, dtype, before=None):
+    """u [T, C], w [C, taps]: y_t = silu(sum_j w[:, j] u_(t - taps + 1 + j)); ``before`` [taps - 1, C]: the rows in front of
+    the first (zeros at the start of a sequence). The projection's result is rounded; what follows is 32-bit."""
     taps = w.shape[1]
-    padded = torch.cat([torch.zeros(taps - 1, u.shape[1]), rnd(u, dtype)])
+    front = torch.zeros(taps - 1, u.shape[1]) if before is None else before
+    padded = torch.cat([front, rnd(u, dtype)])
     y = sum(padded[j:j + u.shape[0]] * w[:, j].float() for j in range(taps))
-    return rnd(silu(y), dtype)
+    return silu(y)
 
 
 def delta_rule(q, k, v, beta, g, state=None):
@@ -158,20 +160,20 @@ def gated_delta(h, m, t, pre, eps, dtype):
     beta = torch.sigmoid(hb @ t[pre + "b"].float().T)
     g = torch.exp(-torch.exp(t[pre + "A_log"].float()) * F.softplus(hb @ t[pre + "a"].float().T + t[pre + "dt_bias"].float()))
     o, _ = delta_rule(q, k, v, beta, g)
-    gate = silu(linear(h, t[pre + "g"], dtype=dtype)).view(T, H, Dv)
+    gate = silu(rnd(linear(h, t[pre + "g"], dtype=dtype), dtype)).view(T, H, Dv)
     y = rms(o, t[pre + "norm"], eps) * gate
-    return linear(y.reshape(T, H * Dv), t[pre + "o"], dtype=dtype)
+    return rnd(linear(y.reshape(T, H * Dv), t[pre + "o"], dtype=dtype), dtype)
 
 
 def parallel_mixer(h, m, t, pre, eps, positions, dtype):
     a = grouped_attention(h, m["left"], t, pre + "left.", eps, positions, dtype)
     b = gated_delta(h, m["right"], t, pre + "right.", eps, dtype)
-    return 0.5 * (rms(a, t[pre + "left.out"], eps) + rms(b, t[pre + "right.out"], eps))
+    return rnd(0.5 * (rms(a, t[pre + "left.out"], eps) + rms(b, t[pre + "right.out"], eps)), dtype)
 
 
 def dense_ff(h, t, pre, dtype):
-    a = rnd(gelu_tanh(linear(h, t[pre + "gate"], dtype=dtype)) * linear(h, t[pre + "up"], dtype=dtype), dtype)
-    return linear(a, t[pre + "down"], dtype=dtype)
+    a = rnd(gelu_tanh(rnd(linear(h, t[pre + "gate"], dtype=dtype), dtype)) * rnd(linear(h, t[pre + "up"], dtype=dtype), dtype), dtype)
+    return rnd(linear(a, t[pre + "down"], dtype=dtype), dtype)
 
 
 def route(h, mlp, t, pre, dtype):
@@ -189,7 +191,7 @@ def expert_ff(h, mlp, t, pre, dtype):
         a = rnd(silu(linear(h, t[p + "gate"], dtype=dtype)) * linear(h, t[p + "up"], dtype=dtype), dtype)
         y = a @ t[p + "down"].float().T
         out = out + y * (weight * (chosen == e)).sum(-1, keepdim=True)
-    return out
+    return rnd(out, dtype)
 
 
 def feed_forward(h, mlp, t, pre, dtype):
