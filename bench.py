@@ -3,7 +3,7 @@ weights, synthetic token ids, on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--dtype bfloat16|float32] [--layers L]
                     [--config CONFIG.json|NAME]      another shape of the architecture (7b, 32b, a file)
-                    [--part all|decode|prefill|offline|mixed7b|preempt32b|modinex|lusolix|gaborax]
+                    [--part all|decode|prefill|offline|mixed7b|preempt32b|modinex|lusolix|gaborax|luzevik]
                     [--part decode --contexts 8192,32768 --batches 8,64]     decode steps over long contexts
 
 A "step" is one decode step of the engine (scheduling, metadata upload, the forward pass and greedy
@@ -19,6 +19,8 @@ of their operations has to move and do), not from formulas of one architecture.
                         (portions of prompts beside decoding requests, budget 2,048), up to 64 at a time
     --part preempt32b   the 32B shape, context 8,192: 64 prompts of 2,048 ids on 8,192 pages of 16, so
                         that growth during decoding evicts requests; reports evictions and tok/s
+    --part luzevik      the Luzevik design at two such sizes (luzevik-1k, luzevik-2k) beside the Lusolix models of those sizes (the
+                        closest design: attention through a shared latent, routed experts, state slots) and the same two Qwen2 models
     --part gaborax      the Gaborax design at two such sizes (gaborax-1k, gaborax-2k) beside the same two Qwen2 models
     --part lusolix      the Lusolix design at two such sizes (lusolix-1k, lusolix-2k) beside the same two Qwen2 models
     --part modinex      the Modinex design at two sizes that resemble a real model's layers (shipped shapes modinex-1k,
@@ -55,6 +57,10 @@ class _Matrices:
 
     def numel(self) -> int:
         return self._n
+
+
+# a design's comparison (--part <design>): the shipped shapes <design>-1k and <design>-2k, each beside these models of its size
+DESIGNS = {"modinex": ("qwen2-like",), "lusolix": ("qwen2-like",), "gaborax": ("qwen2-like",), "luzevik": ("lusolix", "qwen2-like")}
 
 
 def _linears(model):
@@ -102,7 +108,7 @@ def main() -> int:
                     help="captured shapes also try every algorithm the library holds, not only its heuristic's candidates")
     ap.add_argument("--skip-points", action="store_true", help="only the headline batch and the prefill")
     ap.add_argument("--skip-kernels", action="store_true", help="no per-operation kernel trace")
-    ap.add_argument("--part", default="all", choices=["all", "decode", "prefill", "offline", "mixed7b", "preempt32b", "modinex", "lusolix", "gaborax"],
+    ap.add_argument("--part", default="all", choices=["all", "decode", "prefill", "offline", "mixed7b", "preempt32b", "modinex", "lusolix", "gaborax", "luzevik"],
                     help="all: the headline line. decode / prefill: only that (for profiling one of them). offline: "
                          "--requests prompts of --offline-prompt tokens submitted at once. mixed7b / preempt32b: see above")
     ap.add_argument("--requests", type=int, default=None, help="requests of the offline, mixed7b and preempt32b parts")
@@ -149,7 +155,7 @@ def main() -> int:
     # the position tables reach the longest context any engine of this run allows (each engine has its own limit)
     most_positions = max([max_model_len] + sweep + ([] if args.skip_points or args.part != "all" else list(LONG_POINTS)))
     most_positions = min(most_positions, shape.get("max_position_embeddings", most_positions))
-    model = None if args.part in ("modinex", "lusolix", "gaborax") else load_random_model(shape, seed=0, dtype=dtype, device=device, max_positions=most_positions)
+    model = None if args.part in DESIGNS else load_random_model(shape, seed=0, dtype=dtype, device=device, max_positions=most_positions)
     gen = torch.Generator().manual_seed(0)
     vocab = model.head.vocab if model is not None else None
 
@@ -368,12 +374,12 @@ def main() -> int:
                 "config": {**sizes(), "requests": n, "prompt": prompt_len, "gen": gen_tokens, "max_num_seqs": n,
                            "token_budget": 2048, "max_model_len": max_model_len, "block_size": BLOCK_SIZE, "pages": pages}}
 
-    if args.part in ("modinex", "lusolix", "gaborax"):
+    if args.part in DESIGNS:
         # the new design beside the closest existing model at equal size: the functions above measure whatever
         # `model` is, so each shape is loaded in turn
         rows = {}
         for size in ("1k", "2k"):
-            for name in (f"{args.part}-{size}", f"qwen2-like-{size}"):
+            for name in (f"{args.part}-{size}", *(f"{other}-{size}" for other in DESIGNS[args.part])):
                 shape, shape_name = read_shape(name), name
                 model = load_random_model(shape, seed=0, dtype=dtype, device=device, max_positions=most_positions)
                 vocab = model.head.vocab
@@ -391,7 +397,7 @@ def main() -> int:
                 del model
                 model = None
                 torch.cuda.empty_cache()
-        print(json.dumps({"metric": f"{args.part.capitalize()} beside Qwen2 at equal size: prefill of {prompt_len} tokens, decode at batch {args.batch}",
+        print(json.dumps({"metric": f"{args.part.capitalize()} beside {' and '.join(DESIGNS[args.part])} at equal size: prefill of {prompt_len} tokens, decode at batch {args.batch}",
                           "dtype": args.dtype, "prompt": prompt_len, "batch": args.batch, "rows": rows}))
         return 0
     if args.part == "offline":
