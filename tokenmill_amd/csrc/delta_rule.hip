@@ -18,9 +18,10 @@
 // The columns of S are independent of each other: with d_k = S^T k and d_q = S^T q taken on the state as the token finds it,
 //   u = beta (v - g d_k),   o = g d_q + u (k . q),   S <- g S + k u^T
 // is the same recurrence with one round of sums a token instead of two. The scan is dealt over (request, head, 16 columns)
-// wavefronts; a lane keeps a quarter of a column's D rows in registers, and a column's four partial sums are added in a fixed
-// order. A token's result depends on its request's state and tokens only, never on the step's other rows or on how the
-// prompt was cut. Everything that enters the recurrence is 32-bit.
+// blocks; a lane keeps a sixteenth of a column's D rows in registers, and a column's sixteen partial sums are added in a fixed
+// order; a request's rows reach its block through LDS, a tile of tokens at a time. A token's result depends on its
+// request's state and tokens only, never on the step's other rows or on how the prompt was cut. Everything that enters the
+// recurrence is 32-bit.
 #include "common.h"
 #include "api.h"
 
@@ -148,79 +149,121 @@ extern "C" int tm_delta_conv_state(const void* proj, int ld, void* state, const 
 
 // ------------------------------------------------------------------------------------------------ the recurrence
 
-// grid (ceil(Dv / (64 / PARTS)), H, S); a block is one wavefront. PARTS (4, or 8 for keys of more than 128 channels) lanes share
-// a column's rows: lane = column * PARTS + part; part p keeps rows p * R .. p * R + R - 1 of its column, R = ceil(D / PARTS) <= RMAX. The next token's operands are asked for before the
-// current token is worked on. VEC: R is a multiple of 4 and the rows are 16-byte aligned, so a lane's q and k come as float4.
-template <int RMAX, int PARTS, bool VEC>
-__global__ __launch_bounds__(TM_WAVE) void delta_scan_kernel(const float* __restrict__ rows, int ld, float* __restrict__ o,
-                                                            float* __restrict__ state, const int* __restrict__ cu_q_lens,
-                                                            const int* __restrict__ state_slots, int H, int G, int D, int Dv) {
-    const int lane = threadIdx.x, part = lane % PARTS;
-    const int e = blockIdx.x * (TM_WAVE / PARTS) + lane / PARTS;
+#define DR_PARTS 16                         // lanes that share a column's rows: a row of 16 lanes, whose sum the data-parallel moves give
+#define DR_COLS 16                          // columns of a block (four wavefronts with four columns each)
+#define DR_THREADS 256
+#define DR_TT 16                            // tokens of a tile
+
+// The sum over the 16 lanes of a row, in every one of them: neighbours, pairs, the mirrored half row, the mirrored row.
+__device__ __forceinline__ float row16_sum(float v) {
+    v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0xB1, 0xF, 0xF, true));     // quad_perm [1, 0, 3, 2]
+    v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x4E, 0xF, 0xF, true));     // quad_perm [2, 3, 0, 1]
+    v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x141, 0xF, 0xF, true));    // row_half_mirror
+    v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x140, 0xF, 0xF, true));    // row_mirror
+    return v;
+}
+
+// grid (ceil(Dv / 16), H, S); a block is four wavefronts and 16 columns of S. Sixteen lanes share a column's rows: lane =
+// column * 16 + part; part p keeps rows p * R .. p * R + R - 1 of its column, R = ceil(D / 16) <= RMAX, so a token costs a lane
+// 3 R multiply-adds and the chain from token to token is short. The request's rows come through LDS in tiles of 16 tokens, each
+// token's [q | k | beta g k.q . | v of the block's columns] (W = 2 D + 20 floats): the block's threads fetch a tile together,
+// consecutive threads consecutive floats, into registers while the tile before is worked on (CPM: floats of a token a thread
+// fetches at most), and put it down in the other of two buffers. VEC: R is a multiple of 4, so a lane reads its q and k from
+// LDS as float4.
+template <int RMAX, int CPM, bool VEC>
+__global__ __launch_bounds__(DR_THREADS) void delta_scan_kernel(const float* __restrict__ rows, int ld, float* __restrict__ o,
+                                                               float* __restrict__ state, const int* __restrict__ cu_q_lens,
+                                                               const int* __restrict__ state_slots, int H, int G, int D, int Dv) {
+    extern __shared__ __align__(16) float tile_s[];                       // [2][DR_TT][W]
+    const int tid = threadIdx.x, part = tid % DR_PARTS, mine = tid / DR_PARTS;
+    const int e = blockIdx.x * DR_COLS + mine;
     const int h = blockIdx.y, s = blockIdx.z;
     const int g = h / (H / G);
-    const int R = (D + PARTS - 1) / PARTS;
+    const int R = (D + DR_PARTS - 1) / DR_PARTS;
     const int d0 = part * R;
     const bool col = e < Dv;
     const int t0 = cu_q_lens[s], t1 = cu_q_lens[s + 1];
-    if (t1 <= t0) return;
-    const int C = 2 * G * D + H * Dv;
-    const size_t q_at = (size_t)g * D + d0, k_at = (size_t)G * D + (size_t)g * D + d0, v_at = (size_t)2 * G * D + (size_t)h * Dv + (col ? e : 0);
+    if (t1 <= t0) return;                                                 // the whole block
+    const int C = 2 * G * D + H * Dv, W = 2 * D + 4 + DR_COLS;
+    // where in a prepared row the floats come from that this thread fetches of every token (-1: none)
+    int from[CPM];
+#pragma unroll
+    for (int j = 0; j < CPM; ++j) {
+        const int c = tid + DR_THREADS * j;
+        int at = -1;
+        if (c < D) at = g * D + c;
+        else if (c < 2 * D) at = G * D + g * D + (c - D);
+        else if (c == 2 * D) at = C + h;
+        else if (c == 2 * D + 1) at = C + H + h;
+        else if (c == 2 * D + 2) at = C + 2 * H + g;
+        else if (c >= 2 * D + 4 && c < W && blockIdx.x * DR_COLS + (c - 2 * D - 4) < Dv) at = 2 * G * D + h * Dv + blockIdx.x * DR_COLS + (c - 2 * D - 4);
+        from[j] = at;
+    }
+    float held[DR_TT * CPM];
+    auto fetch = [&](int first) {
+#pragma unroll
+        for (int tt = 0; tt < DR_TT; ++tt)
+#pragma unroll
+            for (int j = 0; j < CPM; ++j)
+                held[tt * CPM + j] = (from[j] >= 0 && first + tt < t1) ? rows[(size_t)(first + tt) * ld + from[j]] : 0.f;
+    };
     float* st = state + (((size_t)state_slots[s] * H + h) * D) * Dv + (col ? e : 0);
     float S[RMAX];
 #pragma unroll
     for (int i = 0; i < RMAX; ++i) S[i] = (col && i < R && d0 + i < D) ? st[(size_t)(d0 + i) * Dv] : 0.f;
-    float cq[RMAX], ck[RMAX], nq[RMAX], nk[RMAX];
-    float cv, cb, cg, cx, nv, nb, ng, nx;
-    auto fetch = [&](int t, float* q, float* k, float& v, float& b, float& gd, float& x) {
-        const float* row = rows + (size_t)t * ld;
-        if (VEC) {
+    fetch(t0);
+    int which = 0;
+    for (int first = t0; first < t1; first += DR_TT) {
+        float* cur = tile_s + which * DR_TT * W;
 #pragma unroll
-            for (int i = 0; i < RMAX; i += 4)
-                if (i < R) {
-                    const float4 a = *(const float4*)(row + q_at + i), c = *(const float4*)(row + k_at + i);
-                    q[i] = a.x, q[i + 1] = a.y, q[i + 2] = a.z, q[i + 3] = a.w;
-                    k[i] = c.x, k[i + 1] = c.y, k[i + 2] = c.z, k[i + 3] = c.w;
+        for (int tt = 0; tt < DR_TT; ++tt)
+#pragma unroll
+            for (int j = 0; j < CPM; ++j) {
+                const int c = tid + DR_THREADS * j;
+                if (c < W) cur[tt * W + c] = held[tt * CPM + j];
+            }
+        // every wavefront is done with the tile before the last (this buffer's last use) when it comes here, so one barrier a
+        // tile orders both the stores above against the reads below and the reads of two tiles ago against these stores
+        __syncthreads();
+        if (first + DR_TT < t1) fetch(first + DR_TT);                     // in flight while this tile is worked on
+        const int n = min(DR_TT, t1 - first);
+        float* out = o + ((size_t)first * H + h) * Dv + e;
+        for (int tt = 0; tt < n; ++tt) {
+            const float* row = cur + tt * W;
+            float kk[RMAX];
+            float dk = 0.f, dq = 0.f;
+            if (VEC) {
+#pragma unroll
+                for (int i = 0; i < RMAX; i += 4)
+                    if (i < R) {
+                        const float4 q4 = *(const float4*)(row + d0 + i), k4 = *(const float4*)(row + D + d0 + i);
+                        kk[i] = k4.x, kk[i + 1] = k4.y, kk[i + 2] = k4.z, kk[i + 3] = k4.w;
+                        dk += S[i] * k4.x, dq += S[i] * q4.x;
+                        dk += S[i + 1] * k4.y, dq += S[i + 1] * q4.y;
+                        dk += S[i + 2] * k4.z, dq += S[i + 2] * q4.z;
+                        dk += S[i + 3] * k4.w, dq += S[i + 3] * q4.w;
+                    }
+            } else {
+#pragma unroll
+                for (int i = 0; i < RMAX; ++i) {
+                    const bool in = i < R && d0 + i < D;
+                    kk[i] = in ? row[D + d0 + i] : 0.f;
+                    if (in) {
+                        dk += S[i] * kk[i];
+                        dq += S[i] * row[d0 + i];
+                    }
                 }
-        } else {
-#pragma unroll
-            for (int i = 0; i < RMAX; ++i) {
-                const bool in = i < R && d0 + i < D;
-                q[i] = in ? row[q_at + i] : 0.f;
-                k[i] = in ? row[k_at + i] : 0.f;
             }
+            dk = row16_sum(dk);
+            dq = row16_sum(dq);
+            const float beta = row[2 * D], decay = row[2 * D + 1], kq = row[2 * D + 2], v = row[2 * D + 4 + mine];
+            const float u = beta * (v - decay * dk);
+#pragma unroll
+            for (int i = 0; i < RMAX; ++i)
+                if (i < R) S[i] = decay * S[i] + kk[i] * u;
+            if (col && part == 0) out[(size_t)tt * H * Dv] = decay * dq + u * kq;
         }
-        v = row[v_at];
-        b = row[C + h];
-        gd = row[C + H + h];
-        x = row[C + 2 * H + g];
-    };
-    fetch(t0, cq, ck, cv, cb, cg, cx);
-    for (int t = t0; t < t1; ++t) {
-        fetch(t + 1 < t1 ? t + 1 : t, nq, nk, nv, nb, ng, nx);            // the last token asks for itself again
-        float dk = 0.f, dq = 0.f;
-#pragma unroll
-        for (int i = 0; i < RMAX; ++i)
-            if (i < R) {
-                dk += S[i] * ck[i];
-                dq += S[i] * cq[i];
-            }
-        dk += __shfl_xor(dk, 1, TM_WAVE);
-        dq += __shfl_xor(dq, 1, TM_WAVE);
-        dk += __shfl_xor(dk, 2, TM_WAVE);
-        dq += __shfl_xor(dq, 2, TM_WAVE);
-        if (PARTS == 8) {
-            dk += __shfl_xor(dk, 4, TM_WAVE);
-            dq += __shfl_xor(dq, 4, TM_WAVE);
-        }
-        const float u = cb * (cv - cg * dk);
-#pragma unroll
-        for (int i = 0; i < RMAX; ++i)
-            if (i < R) S[i] = cg * S[i] + ck[i] * u;
-        if (col && part == 0) o[((size_t)t * H + h) * Dv + e] = cg * dq + u * cx;
-#pragma unroll
-        for (int i = 0; i < RMAX; ++i) cq[i] = nq[i], ck[i] = nk[i];
-        cv = nv, cb = nb, cg = ng, cx = nx;
+        which ^= 1;
     }
 #pragma unroll
     for (int i = 0; i < RMAX; ++i)
@@ -233,19 +276,20 @@ extern "C" int tm_delta_scan(const float* rows, int ld, float* o, float* state, 
         H > 65535 || S > 65535 || (long long)ld < 2LL * G * D + (long long)H * Dv + 2 * H + G)
         return TM_ERR_ARG;
     if (S == 0) return TM_OK;
-    const int parts = D > 128 ? 8 : 4, cols = TM_WAVE / parts;
-    const dim3 grid((Dv + cols - 1) / cols, H, S);
-    const int R = (D + parts - 1) / parts;
-    const bool vec = D % (4 * parts) == 0 && ld % 4 == 0 && ((uintptr_t)rows % 16) == 0;
-#define DR_GO(RM, P)                                                                                                            \
-    do {                                                                                                                        \
-        if (vec) delta_scan_kernel<RM, P, true><<<grid, TM_WAVE, 0, stream>>>(rows, ld, o, state, cu_q_lens, state_slots, H, G, D, Dv); \
-        else delta_scan_kernel<RM, P, false><<<grid, TM_WAVE, 0, stream>>>(rows, ld, o, state, cu_q_lens, state_slots, H, G, D, Dv);    \
+    const dim3 grid((Dv + DR_COLS - 1) / DR_COLS, H, S);
+    const int W = 2 * D + 4 + DR_COLS;
+    const size_t lds = (size_t)2 * DR_TT * W * sizeof(float);              // 68 KB at most
+    const bool vec = D % (4 * DR_PARTS) == 0;
+#define DR_GO(RM, CPM_)                                                                                                          \
+    do {                                                                                                                         \
+        auto kernel = vec ? delta_scan_kernel<RM, CPM_, true> : delta_scan_kernel<RM, CPM_, false>;                              \
+        if (lds > 64 * 1024 && hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) \
+            return TM_ERR_LAUNCH;                                                                                                \
+        kernel<<<grid, DR_THREADS, lds, stream>>>(rows, ld, o, state, cu_q_lens, state_slots, H, G, D, Dv);                      \
     } while (0)
-    if (parts == 8) DR_GO(32, 8);
-    else if (R <= 8) DR_GO(8, 4);
-    else if (R <= 16) DR_GO(16, 4);
-    else DR_GO(32, 4);
+    if (D <= 64) DR_GO(4, 1);                       // W <= 148
+    else if (D <= 128) DR_GO(8, 2);                 // W <= 276
+    else DR_GO(16, 3);                              // W <= 532
 #undef DR_GO
     TM_CHECK_LAUNCH();
     return TM_OK;
