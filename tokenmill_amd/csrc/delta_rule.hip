@@ -30,7 +30,24 @@
 
 __device__ __forceinline__ float silu_f32(float z) { return z / (1.0f + expf(-z)); }
 
-// grid T; a block is a token. LDS: C floats (the token's convolved channels).
+// A channel of a token behind the convolution and silu: `taps` rows ending at the token, those before the step's first row from
+// the request's convolution state.
+template <typename T>
+__device__ __forceinline__ float delta_conv_channel(const T* __restrict__ proj, int ld, const T* __restrict__ conv_w,
+                                                    const T* __restrict__ st, int C, int taps, int first, int i, int c) {
+    float acc = 0.f;
+    for (int j = 0; j < taps; ++j) {
+        const int at = i - (taps - 1) + j;                   // < 0: before this step's rows, in the state
+        const float x = at >= 0 ? Elem<T>::load(proj + (size_t)(first + at) * ld + c)
+                                : Elem<T>::load(st + (size_t)(taps - 1 + at) * C + c);
+        acc += Elem<T>::load(conv_w + (size_t)c * taps + j) * x;
+    }
+    return silu_f32(acc);
+}
+
+// grid (T, G + ceil(H Dv / 256)); a block is a token and either one q/k head (a thread a channel of q and of k; the head's three
+// sums by the block's fixed tree) or 256 channels of v; the first block of v also makes the token's step sizes and decays. Few
+// tokens still make many blocks, and a thread's loads are a handful.
 template <typename T>
 __global__ __launch_bounds__(DP_THREADS) void delta_prepare_kernel(const T* __restrict__ proj, int ld, const T* __restrict__ conv_w,
                                                                    const T* __restrict__ conv_state, const float* __restrict__ ba,
@@ -39,51 +56,37 @@ __global__ __launch_bounds__(DP_THREADS) void delta_prepare_kernel(const T* __re
                                                                    const int* __restrict__ slots, const int* __restrict__ seq_of_token,
                                                                    float* __restrict__ out, int ldo, int H, int G, int D, int Dv,
                                                                    int taps, float unit_eps) {
-    extern __shared__ float ch[];
-    const int t = blockIdx.x;
+    __shared__ float red[DP_THREADS / TM_WAVE];
+    const int t = blockIdx.x, unit = blockIdx.y;
     const int s = seq_of_token[t];
     const int first = cu[s], i = t - first;                  // the token's place among its request's rows of this step
     const int C = 2 * G * D + H * Dv;
     const T* st = conv_state + (size_t)slots[s] * (taps - 1) * C;
-    for (int c = threadIdx.x; c < C; c += DP_THREADS) {
-        float acc = 0.f;
-        for (int j = 0; j < taps; ++j) {
-            const int at = i - (taps - 1) + j;               // < 0: before this step's rows, in the state
-            const float x = at >= 0 ? Elem<T>::load(proj + (size_t)(first + at) * ld + c)
-                                    : Elem<T>::load(st + (size_t)(taps - 1 + at) * C + c);
-            acc += Elem<T>::load(conv_w + (size_t)c * taps + j) * x;
-        }
-        ch[c] = silu_f32(acc);
-    }
-    __syncthreads();
     float* o = out + (size_t)t * ldo;
-    const int wave = threadIdx.x / TM_WAVE, lane = threadIdx.x % TM_WAVE;
-    const float q_scale = 1.0f / sqrtf((float)D);
-    for (int g = wave; g < G; g += DP_THREADS / TM_WAVE) {   // a wavefront a q/k head
-        const float* q = ch + g * D;
-        const float* k = ch + G * D + g * D;
-        float sq = 0.f, sk = 0.f, qk = 0.f;
-        for (int d = lane; d < D; d += TM_WAVE) {
-            sq += q[d] * q[d];
-            sk += k[d] * k[d];
-            qk += q[d] * k[d];
+    if (unit < G) {                                          // D <= 256: a thread has one channel of the head's q and one of its k
+        const int c = threadIdx.x;
+        const bool in = c < D;
+        const float q = in ? delta_conv_channel<T>(proj, ld, conv_w, st, C, taps, first, i, unit * D + c) : 0.f;
+        const float k = in ? delta_conv_channel<T>(proj, ld, conv_w, st, C, taps, first, i, G * D + unit * D + c) : 0.f;
+        const float sq = block_sum<DP_THREADS>(q * q, red), sk = block_sum<DP_THREADS>(k * k, red), qk = block_sum<DP_THREADS>(q * k, red);
+        const float iq = (1.0f / sqrtf((float)D)) / sqrtf(sq + unit_eps), ik = 1.0f / sqrtf(sk + unit_eps);
+        if (in) {
+            o[unit * D + c] = q * iq;
+            o[G * D + unit * D + c] = k * ik;
         }
-        sq = wave_sum(sq), sk = wave_sum(sk), qk = wave_sum(qk);
-        const float iq = q_scale / sqrtf(sq + unit_eps), ik = 1.0f / sqrtf(sk + unit_eps);
-        for (int d = lane; d < D; d += TM_WAVE) {
-            o[g * D + d] = q[d] * iq;
-            o[G * D + g * D + d] = k[d] * ik;
+        if (c == 0) o[C + 2 * H + unit] = qk * iq * ik;
+        return;
+    }
+    const int c = 2 * G * D + (unit - G) * DP_THREADS + threadIdx.x;
+    if (c < C) o[c] = delta_conv_channel<T>(proj, ld, conv_w, st, C, taps, first, i, c);
+    if (unit == G)
+        for (int h = threadIdx.x; h < H; h += DP_THREADS) {
+            const float b = ba[(size_t)t * ldba + h];
+            const float a = ba[(size_t)t * ldba + H + h] + dt_bias[h];
+            const float sp = fmaxf(a, 0.f) + log1pf(expf(-fabsf(a)));            // softplus
+            o[C + h] = 1.0f / (1.0f + expf(-b));
+            o[C + H + h] = expf(-expf(a_log[h]) * sp);
         }
-        if (lane == 0) o[C + 2 * H + g] = qk * iq * ik;
-    }
-    for (int c = 2 * G * D + threadIdx.x; c < C; c += DP_THREADS) o[c] = ch[c];
-    for (int h = threadIdx.x; h < H; h += DP_THREADS) {
-        const float b = ba[(size_t)t * ldba + h];
-        const float a = ba[(size_t)t * ldba + H + h] + dt_bias[h];
-        const float sp = fmaxf(a, 0.f) + log1pf(expf(-fabsf(a)));            // softplus
-        o[C + h] = 1.0f / (1.0f + expf(-b));
-        o[C + H + h] = expf(-expf(a_log[h]) * sp);
-    }
 }
 
 extern "C" int tm_delta_prepare(const void* proj, int ld, const void* conv_w, const void* conv_state, const float* ba, int ldba,
@@ -91,22 +94,23 @@ extern "C" int tm_delta_prepare(const void* proj, int ld, const void* conv_w, co
                                 const int* seq_of_token, float* out, int ldo, int T, int H, int G, int D, int Dv, int taps,
                                 float unit_eps, int dtype, hipStream_t stream) {
     if (!proj || !conv_w || !ba || !a_log || !dt_bias || !cu_q_lens || !state_slots || !seq_of_token || !out || T < 0 || H <= 0 ||
-        G <= 0 || H % G || D <= 0 || Dv <= 0 || taps < 1 || taps > DR_MAX_TAPS || (taps > 1 && !conv_state) || ldba < 2 * H ||
-        !(unit_eps > 0.f))
+        G <= 0 || H % G || D <= 0 || D > DP_THREADS || Dv <= 0 || taps < 1 || taps > DR_MAX_TAPS || (taps > 1 && !conv_state) ||
+        ldba < 2 * H || !(unit_eps > 0.f))
         return TM_ERR_ARG;
     const long long C = 2LL * G * D + (long long)H * Dv;
-    if (ld < C || ldo < C + 2 * H + G || C * 4 > 64 * 1024) return TM_ERR_ARG;
+    const long long units = G + ((long long)H * Dv + DP_THREADS - 1) / DP_THREADS;
+    if (ld < C || ldo < C + 2 * H + G || units > 65535) return TM_ERR_ARG;
     if (dtype != TM_F32 && dtype != TM_BF16) return TM_ERR_ARG;
     if (T == 0) return TM_OK;
-    const size_t lds = (size_t)C * sizeof(float);
+    const dim3 grid(T, (unsigned)units);
     if (dtype == TM_F32)
-        delta_prepare_kernel<float><<<T, DP_THREADS, lds, stream>>>((const float*)proj, ld, (const float*)conv_w, (const float*)conv_state,
-                                                                    ba, ldba, a_log, dt_bias, cu_q_lens, state_slots, seq_of_token, out,
-                                                                    ldo, H, G, D, Dv, taps, unit_eps);
+        delta_prepare_kernel<float><<<grid, DP_THREADS, 0, stream>>>((const float*)proj, ld, (const float*)conv_w, (const float*)conv_state,
+                                                                     ba, ldba, a_log, dt_bias, cu_q_lens, state_slots, seq_of_token, out,
+                                                                     ldo, H, G, D, Dv, taps, unit_eps);
     else
-        delta_prepare_kernel<bf16_t><<<T, DP_THREADS, lds, stream>>>((const bf16_t*)proj, ld, (const bf16_t*)conv_w,
-                                                                     (const bf16_t*)conv_state, ba, ldba, a_log, dt_bias, cu_q_lens,
-                                                                     state_slots, seq_of_token, out, ldo, H, G, D, Dv, taps, unit_eps);
+        delta_prepare_kernel<bf16_t><<<grid, DP_THREADS, 0, stream>>>((const bf16_t*)proj, ld, (const bf16_t*)conv_w,
+                                                                      (const bf16_t*)conv_state, ba, ldba, a_log, dt_bias, cu_q_lens,
+                                                                      state_slots, seq_of_token, out, ldo, H, G, D, Dv, taps, unit_eps);
     TM_CHECK_LAUNCH();
     return TM_OK;
 }

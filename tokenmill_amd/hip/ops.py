@@ -1866,7 +1866,7 @@ def moe_experts_weighted(x: torch.Tensor, routed, weight: torch.Tensor, w_up: to
 # -------------------------------------------------------------------------------------------- the gated delta rule
 
 DELTA_MAX_KEY_DIM = 256
-DELTA_MAX_CHANNELS = 16384          # convolved channels of a token (q | k | v): what a block keeps in LDS
+DELTA_MAX_CHANNELS = 1 << 22        # convolved channels of a token (q | k | v)
 
 
 def delta_row_width(H: int, G: int, D: int, Dv: int) -> int:
