@@ -221,7 +221,9 @@ int tm_delta_prepare(const void* proj, int ld, const void* conv_w, const void* c
 int tm_delta_conv_state(const void* proj, int ld, void* state, const int* cu_q_lens, const int* state_slots, int S, int C, int taps,
                         int dtype, hipStream_t stream);
 int tm_delta_scan(const float* rows, int ld, float* o, float* state, const int* cu_q_lens, const int* state_slots, int S, int H, int G,
-                  int D, int Dv, hipStream_t stream);
+                  int D, int Dv, int row_dv, int use_v, hipStream_t stream);
+int tm_delta_combine(const float* trans, const float* local, float* start, float* state, const int* state_slots, const int* first_seg,
+                     int S, int H, int D, int Dv, hipStream_t stream);
 int tm_pair_norm_mean(const void* a, const void* b, const float* wa, const float* wb, void* out, int T, int W, float eps, int dtype,
                       hipStream_t stream);
 int tm_gelu_mul(const void* gu, void* out, int dtype, int T, int I, hipStream_t stream);

@@ -13,6 +13,8 @@
 //                        as one 32-bit row [q (G D) | k (G D) | v (H Dv) | beta (H) | g (H) | k.q (G)]
 //   tm_delta_conv_state  then the convolution state becomes the last taps - 1 projection rows the request has seen
 //   tm_delta_scan        the recurrence over those rows; writes o in 32-bit
+//   tm_delta_combine     chains the segments of a long portion (each scanned from zero and from the identity) into every
+//                        segment's true start state
 //   tm_pair_norm_mean    out = (rms_norm(a; wa) + rms_norm(b; wb)) / 2: two sublayers side by side, each normed over the width
 //
 // The columns of S are independent of each other: with d_k = S^T k and d_q = S^T q taken on the state as the token finds it,
@@ -173,11 +175,13 @@ __device__ __forceinline__ float row16_sum(float v) {
 // token's [q | k | beta g k.q . | v of the block's columns] (W = 2 D + 20 floats): the block's threads fetch a tile together,
 // consecutive threads consecutive floats, into registers while the tile before is worked on (CPM: floats of a token a thread
 // fetches at most), and put it down in the other of two buffers. VEC: R is a multiple of 4, so a lane reads its q and k from
-// LDS as float4.
+// LDS as float4. o null: only the states are wanted. use_v 0: the values count as zero and the state's Dv columns need not be the
+// rows' row_dv (a scan from the identity gives the product of the tokens' transitions g (I - beta k k^T)).
 template <int RMAX, int CPM, bool VEC>
 __global__ __launch_bounds__(DR_THREADS) void delta_scan_kernel(const float* __restrict__ rows, int ld, float* __restrict__ o,
                                                                float* __restrict__ state, const int* __restrict__ cu_q_lens,
-                                                               const int* __restrict__ state_slots, int H, int G, int D, int Dv) {
+                                                               const int* __restrict__ state_slots, int H, int G, int D, int Dv,
+                                                               int row_dv, int use_v) {
     extern __shared__ __align__(16) float tile_s[];                       // [2][DR_TT][W]
     const int tid = threadIdx.x, part = tid % DR_PARTS, mine = tid / DR_PARTS;
     const int e = blockIdx.x * DR_COLS + mine;
@@ -188,7 +192,7 @@ __global__ __launch_bounds__(DR_THREADS) void delta_scan_kernel(const float* __r
     const bool col = e < Dv;
     const int t0 = cu_q_lens[s], t1 = cu_q_lens[s + 1];
     if (t1 <= t0) return;                                                 // the whole block
-    const int C = 2 * G * D + H * Dv, W = 2 * D + 4 + DR_COLS;
+    const int C = 2 * G * D + H * row_dv, W = 2 * D + 4 + DR_COLS;
     // where in a prepared row the floats come from that this thread fetches of every token (-1: none)
     int from[CPM];
 #pragma unroll
@@ -200,7 +204,8 @@ __global__ __launch_bounds__(DR_THREADS) void delta_scan_kernel(const float* __r
         else if (c == 2 * D) at = C + h;
         else if (c == 2 * D + 1) at = C + H + h;
         else if (c == 2 * D + 2) at = C + 2 * H + g;
-        else if (c >= 2 * D + 4 && c < W && blockIdx.x * DR_COLS + (c - 2 * D - 4) < Dv) at = 2 * G * D + h * Dv + blockIdx.x * DR_COLS + (c - 2 * D - 4);
+        else if (use_v && c >= 2 * D + 4 && c < W && blockIdx.x * DR_COLS + (c - 2 * D - 4) < Dv)
+            at = 2 * G * D + h * row_dv + blockIdx.x * DR_COLS + (c - 2 * D - 4);
         from[j] = at;
     }
     float held[DR_TT * CPM];
@@ -265,7 +270,7 @@ __global__ __launch_bounds__(DR_THREADS) void delta_scan_kernel(const float* __r
 #pragma unroll
             for (int i = 0; i < RMAX; ++i)
                 if (i < R) S[i] = decay * S[i] + kk[i] * u;
-            if (col && part == 0) out[(size_t)tt * H * Dv] = decay * dq + u * kq;
+            if (o && col && part == 0) out[(size_t)tt * H * Dv] = decay * dq + u * kq;
         }
         which ^= 1;
     }
@@ -275,9 +280,10 @@ __global__ __launch_bounds__(DR_THREADS) void delta_scan_kernel(const float* __r
 }
 
 extern "C" int tm_delta_scan(const float* rows, int ld, float* o, float* state, const int* cu_q_lens, const int* state_slots, int S,
-                             int H, int G, int D, int Dv, hipStream_t stream) {
-    if (!rows || !o || !state || !cu_q_lens || !state_slots || S < 0 || H <= 0 || G <= 0 || H % G || D <= 0 || D > 256 || Dv <= 0 ||
-        H > 65535 || S > 65535 || (long long)ld < 2LL * G * D + (long long)H * Dv + 2 * H + G)
+                             int H, int G, int D, int Dv, int row_dv, int use_v, hipStream_t stream) {
+    if (!rows || !state || !cu_q_lens || !state_slots || S < 0 || H <= 0 || G <= 0 || H % G || D <= 0 || D > 256 || Dv <= 0 ||
+        row_dv <= 0 || (use_v && row_dv != Dv) || (o && !use_v) || H > 65535 || S > 65535 ||
+        (long long)ld < 2LL * G * D + (long long)H * row_dv + 2 * H + G)
         return TM_ERR_ARG;
     if (S == 0) return TM_OK;
     const dim3 grid((Dv + DR_COLS - 1) / DR_COLS, H, S);
@@ -289,12 +295,92 @@ extern "C" int tm_delta_scan(const float* rows, int ld, float* o, float* state, 
         auto kernel = vec ? delta_scan_kernel<RM, CPM_, true> : delta_scan_kernel<RM, CPM_, false>;                              \
         if (lds > 64 * 1024 && hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess) \
             return TM_ERR_LAUNCH;                                                                                                \
-        kernel<<<grid, DR_THREADS, lds, stream>>>(rows, ld, o, state, cu_q_lens, state_slots, H, G, D, Dv);                      \
+        kernel<<<grid, DR_THREADS, lds, stream>>>(rows, ld, o, state, cu_q_lens, state_slots, H, G, D, Dv, row_dv, use_v);       \
     } while (0)
     if (D <= 64) DR_GO(4, 1);                       // W <= 148
     else if (D <= 128) DR_GO(8, 2);                 // W <= 276
     else DR_GO(16, 3);                              // W <= 532
 #undef DR_GO
+    TM_CHECK_LAUNCH();
+    return TM_OK;
+}
+
+// A prompt in segments: the recurrence is linear in the state, S_end = M S_start + B over any run of tokens, with M the product
+// of the tokens' transitions (a scan from the identity without values) and B what the run builds from a zero state. This chains
+// the segments of every request: start[j] = S; S <- trans[j] S + local[j], from the request's own state, which becomes the last S.
+// grid (ceil(Dv / 16), H, requests); a block keeps 16 columns of S in LDS. A thread owns one row d of the new S and NC of the 16
+// columns (DP: D rounded up to 64, 128 or 256; 256 / DP groups of threads share the columns): it streams its row of M once,
+// sixteen bytes at a time, against the columns it reads from LDS with all its wavefront; every sum over d' in ascending order.
+template <int DP>
+__global__ __launch_bounds__(DR_THREADS) void delta_combine_kernel(const float* __restrict__ trans, const float* __restrict__ local,
+                                                                  float* __restrict__ start, float* __restrict__ state,
+                                                                  const int* __restrict__ state_slots, const int* __restrict__ first_seg,
+                                                                  int H, int D, int Dv) {
+    extern __shared__ __align__(16) float col_s[];                        // [D][16]
+    constexpr int NC = DR_COLS * DP / DR_THREADS;                         // columns of a thread: 4, 8 or 16
+    const int d = threadIdx.x % DP, c0 = threadIdx.x / DP * NC;
+    const int e0 = blockIdx.x * DR_COLS;
+    const int h = blockIdx.y, s = blockIdx.z;
+    float* st = state + (((size_t)state_slots[s] * H + h) * D) * Dv;
+    for (int idx = threadIdx.x; idx < D * DR_COLS; idx += DR_THREADS) {
+        const int dd = idx / DR_COLS, e = e0 + idx % DR_COLS;
+        col_s[idx] = e < Dv ? st[(size_t)dd * Dv + e] : 0.f;
+    }
+    __syncthreads();
+    for (int seg = first_seg[s]; seg < first_seg[s + 1]; ++seg) {
+        const size_t at = ((size_t)seg * H + h) * D;
+        for (int idx = threadIdx.x; idx < D * DR_COLS; idx += DR_THREADS) {
+            const int dd = idx / DR_COLS, e = e0 + idx % DR_COLS;
+            if (e < Dv) start[(at + dd) * Dv + e] = col_s[idx];
+        }
+        float acc[NC];
+#pragma unroll
+        for (int j = 0; j < NC; ++j) acc[j] = (d < D && e0 + c0 + j < Dv) ? local[(at + d) * Dv + e0 + c0 + j] : 0.f;
+        if (d < D) {
+            const float* m = trans + (at + d) * D;
+            if (D % 4 == 0) {
+#pragma unroll 4
+                for (int k = 0; k < D; k += 4) {
+                    const float4 m4 = *(const float4*)(m + k);
+#pragma unroll
+                    for (int j = 0; j < NC; ++j) {
+                        acc[j] += m4.x * col_s[k * DR_COLS + c0 + j];
+                        acc[j] += m4.y * col_s[(k + 1) * DR_COLS + c0 + j];
+                        acc[j] += m4.z * col_s[(k + 2) * DR_COLS + c0 + j];
+                        acc[j] += m4.w * col_s[(k + 3) * DR_COLS + c0 + j];
+                    }
+                }
+            } else {
+                for (int k = 0; k < D; ++k) {
+                    const float mk = m[k];
+#pragma unroll
+                    for (int j = 0; j < NC; ++j) acc[j] += mk * col_s[k * DR_COLS + c0 + j];
+                }
+            }
+        }
+        __syncthreads();                                                  // every row has read the old columns
+        if (d < D)
+#pragma unroll
+            for (int j = 0; j < NC; ++j) col_s[d * DR_COLS + c0 + j] = acc[j];
+        __syncthreads();
+    }
+    for (int idx = threadIdx.x; idx < D * DR_COLS; idx += DR_THREADS) {
+        const int dd = idx / DR_COLS, e = e0 + idx % DR_COLS;
+        if (e < Dv) st[(size_t)dd * Dv + e] = col_s[idx];
+    }
+}
+
+extern "C" int tm_delta_combine(const float* trans, const float* local, float* start, float* state, const int* state_slots,
+                                const int* first_seg, int S, int H, int D, int Dv, hipStream_t stream) {
+    if (!trans || !local || !start || !state || !state_slots || !first_seg || S < 0 || H <= 0 || H > 65535 || S > 65535 || D <= 0 ||
+        D > DR_THREADS || Dv <= 0)
+        return TM_ERR_ARG;
+    if (S == 0) return TM_OK;
+    const dim3 grid((Dv + DR_COLS - 1) / DR_COLS, H, S);
+    const size_t lds = (size_t)D * DR_COLS * sizeof(float);
+    if (D <= 64) delta_combine_kernel<64><<<grid, DR_THREADS, lds, stream>>>(trans, local, start, state, state_slots, first_seg, H, D, Dv);
+    else if (D <= 128) delta_combine_kernel<128><<<grid, DR_THREADS, lds, stream>>>(trans, local, start, state, state_slots, first_seg, H, D, Dv);
+    else delta_combine_kernel<256><<<grid, DR_THREADS, lds, stream>>>(trans, local, start, state, state_slots, first_seg, H, D, Dv);
     TM_CHECK_LAUNCH();
     return TM_OK;
 }

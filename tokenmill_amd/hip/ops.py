@@ -1928,24 +1928,48 @@ def delta_conv_state(proj: torch.Tensor, C: int, conv_state: torch.Tensor, cu_q_
                                          c_int(conv_state.shape[1] + 1), c_int(code(proj.dtype)), _stream()), "delta_conv_state")
 
 
-def delta_scan(rows: torch.Tensor, o: torch.Tensor, state: torch.Tensor, cu_q_lens: torch.Tensor, state_slots: torch.Tensor,
-               num_seqs: int, H: int, G: int, D: int, Dv: int) -> torch.Tensor:
+def delta_scan(rows: torch.Tensor, o: torch.Tensor | None, state: torch.Tensor, cu_q_lens: torch.Tensor, state_slots: torch.Tensor,
+               num_seqs: int, H: int, G: int, D: int, Dv: int, transitions_of: int | None = None) -> torch.Tensor | None:
     """The recurrence over the rows of ``delta_prepare``, request by request in the order of the step's rows:
     S <- g S; u = beta (v - S^T k); S <- S + k u^T; o = S^T q. state float32 [slots, H, D, Dv] (row state_slots[s] is read and
-    written); o float32 [T, H * Dv]."""
+    written); o float32 [T, H * Dv], or None where only the states are wanted. ``transitions_of`` = the rows' value size: the
+    values count as zero and the state has ``Dv`` columns of its own (from the identity, Dv = D, a run of tokens leaves the
+    product of its transitions g (I - beta k k^T))."""
     _gpu(rows, o, state, cu_q_lens, state_slots)
     T = rows.shape[0]
-    _need(rows.dtype == torch.float32 and rows.dim() == 2 and rows.is_contiguous() and rows.shape[1] >= 2 * G * D + H * Dv + 2 * H + G,
+    row_dv = Dv if transitions_of is None else transitions_of
+    _need(rows.dtype == torch.float32 and rows.dim() == 2 and rows.is_contiguous() and rows.shape[1] >= 2 * G * D + H * row_dv + 2 * H + G,
           "delta_scan: rows are those of delta_prepare")
-    _need(o.dtype == torch.float32 and o.is_contiguous() and tuple(o.shape) == (T, H * Dv), f"delta_scan: o is float32 [{T}, {H * Dv}]")
+    if o is not None:
+        _need(transitions_of is None, "delta_scan: a scan without values has no results")
+        _need(o.dtype == torch.float32 and o.is_contiguous() and tuple(o.shape) == (T, H * Dv), f"delta_scan: o is float32 [{T}, {H * Dv}]")
     _need(state.dtype == torch.float32 and state.is_contiguous() and tuple(state.shape[1:]) == (H, D, Dv),
           f"delta_scan: state is float32 [slots, {H}, {D}, {Dv}]")
     _need(H % G == 0 and 0 < D <= DELTA_MAX_KEY_DIM, "delta_scan: sizes the kernel does not take")
     _ints(cu_q_lens, num_seqs + 1, "cu_q_lens")
     _ints(state_slots, num_seqs, "state_slots")
     _check(library().tm_delta_scan(_p(rows), c_int(rows.shape[1]), _p(o), _p(state), _p(cu_q_lens), _p(state_slots), c_int(num_seqs),
-                                   c_int(H), c_int(G), c_int(D), c_int(Dv), _stream()), "delta_scan")
+                                   c_int(H), c_int(G), c_int(D), c_int(Dv), c_int(row_dv), c_int(0 if transitions_of is not None else 1),
+                                   _stream()), "delta_scan")
     return o
+
+
+def delta_combine(trans: torch.Tensor, local: torch.Tensor, start: torch.Tensor, state: torch.Tensor, state_slots: torch.Tensor,
+                  first_seg: torch.Tensor, num_seqs: int) -> None:
+    """Chains the segments of every request: start[j] = S, S <- trans[j] S + local[j] for its segments j = first_seg[s] ..
+    first_seg[s + 1] - 1 in order, from S = state[state_slots[s]], which becomes the last S. trans float32 [n, H, D, D], local and
+    start [n, H, D, Dv], state [slots, H, D, Dv]."""
+    _gpu(trans, local, start, state, state_slots, first_seg)
+    n, H, D, Dv = local.shape
+    for name, t, shape in (("trans", trans, (n, H, D, D)), ("local", local, (n, H, D, Dv)), ("start", start, (n, H, D, Dv))):
+        _need(t.dtype == torch.float32 and t.is_contiguous() and tuple(t.shape) == shape, f"delta_combine: {name} is float32 {list(shape)}")
+    _need(state.dtype == torch.float32 and state.is_contiguous() and tuple(state.shape[1:]) == (H, D, Dv),
+          f"delta_combine: state is float32 [slots, {H}, {D}, {Dv}]")
+    _need(0 < D <= DELTA_MAX_KEY_DIM, "delta_combine: sizes the kernel does not take")
+    _ints(state_slots, num_seqs, "state_slots")
+    _ints(first_seg, num_seqs + 1, "first_seg")
+    _check(library().tm_delta_combine(_p(trans), _p(local), _p(start), _p(state), _p(state_slots), _p(first_seg), c_int(num_seqs), c_int(H),
+                                      c_int(D), c_int(Dv), _stream()), "delta_combine")
 
 
 def pair_norm_mean(a: torch.Tensor, b: torch.Tensor, wa: torch.Tensor, wb: torch.Tensor, out: torch.Tensor, eps: float) -> torch.Tensor:

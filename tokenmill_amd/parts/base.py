@@ -119,6 +119,30 @@ class StepContext:
     prefill_tiles: torch.Tensor | None = None
 
 
+def step_segments(step: StepContext, size: int, device):
+    """The step's portions cut into segments of at most ``size`` rows, for a recurrence that scans segments side by side:
+    (first row of each segment int32 [n + 1], 0..n-1 int32 [n], first segment of each request int32 [S + 1], n), made once per
+    step and size from the host's view of its portions and shared by the step's layers."""
+    made = getattr(step, "_segments", None)
+    if made is None:
+        made = step._segments = {}
+    if size not in made:
+        cu, first, row = [0], [0], 0
+        for n in step.q_lens:
+            for lo in range(0, n, size):
+                row += min(size, n - lo)
+                cu.append(row)
+            first.append(len(cu) - 1)
+        # q_lens covers the step's real requests; a step laid out in a padded shape is never segmented (its portions belong
+        # to a model without state)
+        if len(first) != step.num_seqs + 1 or row != step.num_tokens:
+            raise ValueError("the step's portions do not cover its rows: it cannot be cut into segments")
+        n_seg = len(cu) - 1
+        flat = torch.tensor(cu + list(range(n_seg)) + first, dtype=torch.int32).to(device)
+        made[size] = (flat[:n_seg + 1], flat[n_seg + 1:2 * n_seg + 1], flat[2 * n_seg + 1:], n_seg)
+    return made[size]
+
+
 # ------------------------------------------------------------------------------------------------
 # the part interfaces
 # ------------------------------------------------------------------------------------------------

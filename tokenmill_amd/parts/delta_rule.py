@@ -19,7 +19,7 @@ import torch
 
 from tokenmill_amd import profiling
 from tokenmill_amd.hip import ops
-from tokenmill_amd.parts.base import LayerCacheSpec, Mixer, StateSpec, StateView, StepContext, as_tensor
+from tokenmill_amd.parts.base import LayerCacheSpec, Mixer, StateSpec, StateView, StepContext, as_tensor, step_segments
 from tokenmill_amd.parts.linear import Linear
 from tokenmill_amd.weights.loader import TensorSpec
 
@@ -122,7 +122,32 @@ class GatedDeltaRule(Mixer):
                               step.seq_of_token, step.num_seqs, rows, H, G, D, Dv, UNIT_EPS)
             if conv_state is not None:
                 ops.delta_conv_state(proj, self.channels, conv_state, step.cu_q_lens, step.state_slots, step.num_seqs)
-            ops.delta_scan(rows, o, matrices, step.cu_q_lens, step.state_slots, step.num_seqs, H, G, D, Dv)
+            self._scan(rows, o, matrices, step)
             ops.gla_out_gate(o, proj[:, self.channels:], self.norm_w, y, H, Dv, self.norm_eps)
         with profiling.label("o_proj", lambda: self.o.cost(T)):
             return self.o.forward(y)
+
+    # Rows of a request's portion from which the recurrence runs in segments of this many rows (see ``_scan``)
+    SEGMENT = 128
+
+    def _scan(self, rows, o, matrices, step: StepContext) -> None:
+        """The recurrence over the step's rows. A step whose longest portion is short (single tokens, small portions) is one
+        scan from the requests' states. A long portion is cut into segments of ``SEGMENT`` rows: the recurrence is linear in
+        the state, S_end = M S_start + B over any run of tokens, so every segment is first scanned twice side by side with all
+        others, from a zero state (B: what its own rows build) and, without values, from the identity (M: the product of its
+        tokens' transitions g (I - beta k k^T)); a chain over the segments gives each segment's true start state and the
+        request's new state; and a third scan of all segments from those gives the results. Three scans that fill the chip and
+        a short chain of small products, instead of one chain over every token. The sums of a token's result are then ordered
+        otherwise than in the plain chain: the two agree up to 32-bit rounding."""
+        H, G, D, Dv = self.num_heads, self.num_kv_heads, self.key_dim, self.value_dim
+        if step.max_q_len < 2 * self.SEGMENT:
+            ops.delta_scan(rows, o, matrices, step.cu_q_lens, step.state_slots, step.num_seqs, H, G, D, Dv)
+            return
+        cu_seg, ids, first, n_seg = step_segments(step, self.SEGMENT, rows.device)
+        local = torch.zeros((n_seg, H, D, Dv), dtype=torch.float32, device=rows.device)
+        ops.delta_scan(rows, None, local, cu_seg, ids, n_seg, H, G, D, Dv)
+        trans = torch.eye(D, dtype=torch.float32, device=rows.device).expand(n_seg, H, D, D).contiguous()
+        ops.delta_scan(rows, None, trans, cu_seg, ids, n_seg, H, G, D, D, transitions_of=Dv)
+        start = torch.empty_like(local)
+        ops.delta_combine(trans, local, start, matrices, step.state_slots, first, step.num_seqs)
+        ops.delta_scan(rows, o, start, cu_seg, ids, n_seg, H, G, D, Dv)

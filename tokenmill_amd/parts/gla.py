@@ -18,7 +18,7 @@ import torch
 
 from tokenmill_amd import profiling
 from tokenmill_amd.hip import ops
-from tokenmill_amd.parts.base import Mixer, StateSpec, StateView, StepContext, as_tensor
+from tokenmill_amd.parts.base import Mixer, StateSpec, StateView, StepContext, as_tensor, step_segments
 from tokenmill_amd.parts.linear import Linear
 from tokenmill_amd.weights.loader import TensorSpec
 
@@ -149,22 +149,6 @@ class GatedLinearAttention(Mixer):
         ops.gla_scan(proj, 0, ks, 2 * ks, decay, o, start, cu_seg, ids, n_seg, H, D, Dv, scale)
 
     def _segments(self, step: StepContext, device):
-        """(first row of each segment [n + 1], 0..n-1, first segment of each request [S + 1], n) on the device, made
-        once per step from the host's view of its portions and shared by the step's gla layers."""
-        made = getattr(step, "_gla_segments", None)
-        if made is None or made[0] != self.SEGMENT:
-            cu, first, row = [0], [0], 0
-            for n in step.q_lens:
-                for lo in range(0, n, self.SEGMENT):
-                    row += min(self.SEGMENT, n - lo)
-                    cu.append(row)
-                first.append(len(cu) - 1)
-            # q_lens covers the step's real requests; a step laid out in a padded shape is never segmented (its
-            # portions belong to a model without state)
-            if len(first) != step.num_seqs + 1 or row != step.num_tokens:
-                raise ValueError("the step's portions do not cover its rows: it cannot be cut into segments")
-            n_seg = len(cu) - 1
-            flat = torch.tensor(cu + list(range(n_seg)) + first, dtype=torch.int32).to(device)
-            made = (self.SEGMENT, flat[:n_seg + 1], flat[n_seg + 1:2 * n_seg + 1], flat[2 * n_seg + 1:], n_seg)
-            step._gla_segments = made
-        return made[1:]
+        """(first row of each segment [n + 1], 0..n-1, first segment of each request [S + 1], n) on the device, made once per step
+        and shared by the step's layers."""
+        return step_segments(step, self.SEGMENT, device)
