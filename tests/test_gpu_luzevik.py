@@ -316,7 +316,8 @@ def test_gated_delta_rule_whole_in_portions_token_by_token_and_beside_another(dt
     mixer = GatedDeltaRule(64, H, G_, D, Dv, taps, 1e-5)
     w = _random_weights(mixer, dt, 0.25)
     m = {"heads": H, "kv_heads": G_, "dim": D, "vdim": Dv, "conv": taps}
-    T = 150
+    T = 300                                                # whole, the portion is scanned in segments; in pieces, as one chain
+    assert T >= 2 * mixer.SEGMENT > T - 113
     x = q(torch.randn(T, 64), dt)
     want = q(P.gated_delta(x, m, w, "a.", 1e-5, dt), dt)
     pools, manager, runner = _alone(mixer, dt)
