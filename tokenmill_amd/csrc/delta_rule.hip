@@ -22,8 +22,9 @@
 // is the same recurrence with one round of sums a token instead of two. The scan is dealt over (request, head, 16 columns)
 // blocks; a lane keeps a sixteenth of a column's D rows in registers, and a column's sixteen partial sums are added in a fixed
 // order; a request's rows reach its block through LDS, a tile of tokens at a time. A token's result depends on its
-// request's state and tokens only, never on the step's other rows or on how the prompt was cut. Everything that enters the
-// recurrence is 32-bit.
+// request's state and tokens only, never on the step's other rows; how the prompt was cut changes it by 32-bit rounding at
+// most (a long portion is scanned in segments, whose sums are ordered otherwise than the plain chain's). Everything that
+// enters the recurrence is 32-bit.
 #include "common.h"
 #include "api.h"
 
